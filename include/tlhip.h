@@ -237,6 +237,62 @@ int tl_model_batch_decode(tl_model* m, int n, const int* tokens_host, const int*
                           float* logits_host, int* next_tokens_host);
 int tl_model_batch_generate_greedy(tl_model* m, int n, const int* first_tokens_host, const int* start_pos_host,
                                    const int* seq_idx_host, int n_steps, int* out_ids_host);
+/* ---- layer-list models: a decoder described layer by layer instead of by the fixed Llama block. No counterpart in the
+ *      reference (its only model is the Llama block). Such a model lives behind the same tl_model handle: tl_model_finalize,
+ *      tl_model_reset_kv, tl_model_decode, tl_model_generate_greedy / _sampled, tl_model_prefill, tl_model_set_prefill
+ *      (terms 1 = bf16 activations in the chunk GEMMs, 3 = FP32-grade), tl_model_device_ptr, tl_model_bytes_per_token and
+ *      tl_model_free work as for a Llama model; the multi-sequence and tensor-parallel entry points refuse it. Weights are
+ *      bf16 matrices [out][in] and stay bf16 in HBM; the residual stream, norms, router, scores and caches are FP32. ------ */
+enum tl_mixer_kind { TL_MIXER_SWA = 0 };            /* sliding-window attention, no rotation, key size != value size allowed */
+enum tl_mlp_kind { TL_MLP_NONE = 0, TL_MLP_MOE = 1 }; /* no feed-forward | routed experts (+ optional shared expert) */
+typedef struct tl_layer_spec {
+  int mixer;                /* tl_mixer_kind */
+  int heads, kv_heads;      /* query heads, key/value heads (query head h reads head h / (heads / kv_heads)) */
+  int dim, vdim;            /* per-head query/key size, value size */
+  int window;               /* position i sees j with 0 <= i - j < window; <= 0: every j <= i */
+  float scale;              /* score = (q . k) * scale */
+  int qk_norm;              /* 1: RMS norm over the WHOLE q and the whole k projection, plain weights */
+  int v_mix;                /* 1: v <- (1 - lambda) v + lambda v_first, v_first = the first such layer's values of the token */
+  int mlp;                  /* tl_mlp_kind */
+  int experts, top;         /* routed experts, experts per token (weights: softmax over the chosen logits) */
+  int expert_ff;            /* y = g * sigmoid(act_alpha * g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit) */
+  float expert_limit;
+  int shared_ff;            /* 0: no shared expert */
+  float shared_limit;
+  float act_alpha;
+} tl_layer_spec;
+typedef struct tl_stack_config {
+  int width, vocab, n_layers;
+  int max_positions;        /* rows of every layer's key/value cache */
+  float norm_eps;           /* every norm: x / sqrt(mean(x^2) + eps); block norms and the embedding / final norm use (1 + w) */
+  const tl_layer_spec* layers;
+} tl_stack_config;
+/* the operators such a model is built from, callable on their own (all FP32 in and out, weights bf16 [rows][cols]):
+ * Y[T][rows] = X[T][cols] W^T; terms 1 / 3 = MFMA GEMM with bf16-rounded / three-term-split activations, 0 = FP32 GEMV (T = 1) */
+int tl_dense_matmul(const void* w_bf16_dev, int rows, int cols, const float* x_dev, float* y_dev, int num_tokens, int terms,
+                    void* stream);
+/* q [T][heads * dim] at positions start_pos.. against caches K [*][kv_heads * dim], V [*][kv_heads * vdim] that already hold
+ * those positions: softmax((q . k) * scale) over the keys j with 0 <= i - j < window (window <= 0: all j <= i) */
+int tl_swa_attention(const float* q_dev, const float* k_cache_dev, const float* v_cache_dev, float* out_dev, int num_tokens,
+                     int start_pos, int heads, int kv_heads, int dim, int vdim, int window, float scale, void* stream);
+/* x[t] += y[t] / sqrt(mean(y[t]^2) + eps) * (1 + weight) */
+int tl_resid_rmsnorm(float* x_dev, const float* y_dev, const float* weight_dev, int num_tokens, int width, float eps, void* stream);
+/* router: logits = W x + bias (FP32); ids [T][top] = the largest logits first (equal: lower index), weights = softmax over them */
+int tl_moe_route(const float* x_dev, int num_tokens, int width, const void* w_bf16_dev, const float* bias_dev, int experts,
+                 int top, int* ids_dev, float* weights_dev, void* stream);
+/* out[r][i] = g * sigmoid(alpha * g) * (u + 1), g = min(in[r][i], limit), u = clamp(in[r][ff + i], -limit, limit) */
+int tl_glu_clamp(const float* gate_up_dev, int rows, int ff, float limit, float alpha, float* out_dev, void* stream);
+int tl_model_create_stack(const tl_stack_config* cfg, tl_model** out);
+/* tensors by checkpoint name: embed, embed.norm, final.norm, head, l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,q.norm,k.norm,vmix},
+ * l<i>.mlp.router, l<i>.mlp.router.b, l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down}. type: TL_BF16 (matrices and
+ * vectors) or TL_F32 (vectors). */
+int tl_model_set_tensor_named(tl_model* m, const char* name, int type, const long long* shape, int ndim, const void* host_data);
+/* a prompt, or a portion of one, at positions start_pos..: logits of the token rows listed in rows_host (ascending; NULL: the
+ * last token when n_rows == 1, all tokens when n_rows == num_tokens) -> logits_host[n_rows][vocab]. The cache keeps what
+ * earlier calls wrote: portions may be cut anywhere. */
+int tl_model_prefill_rows(tl_model* m, const int* tokens_host, int num_tokens, int start_pos, const int* rows_host, int n_rows,
+                          float* logits_host);
+
 /* tensor-parallel wiring (one process per GPU): RCCL communicator over xGMI; unique_id is the ncclUniqueId (128 bytes)
  * produced by tl_tp_unique_id on rank 0 and broadcast by the host (torch.distributed). Call tl_model_tp_init on every
  * rank before tl_model_finalize: the decode step (incl. its 2 all-reduces per layer and the logits all-gather) is

@@ -44,6 +44,12 @@ int tl_model_bench_kernel(tl_model* m, int kind, int iters, int warmup, float* a
  * in this process: lets a test prove which kernel formed a result. */
 int tl_debug_gemm_px_launches(long long* count_out);
 
+/* Parity hook for layer-list models (no counterpart in the reference): cb(ctx, layer, x_dev, num_tokens, width) is called after
+ * every layer of every forward pass, the stream synchronised, with the residual stream on the device. NULL switches it off.
+ * With the hook set the decode step must run eagerly (TL_NO_GRAPH=1 at finalize): a captured step cannot call back. */
+typedef void (*tl_layer_hook_fn)(void* ctx, int layer, const float* x_dev, int num_tokens, int width);
+int tl_model_debug_layer_hook(tl_model* m, tl_layer_hook_fn cb, void* ctx);
+
 /* ---- libtlhip_tools.so (csrc/tl_stream.hip; built beside libtlhip.so, not part of it): a measured negative result kept
  * for the record -- the persistent ring-loader engine of round 2. */
 /* Measurement / parity hook (no counterpart in the reference): y_i = W_i x through the ring-loader engine (tl_stream.hip),

@@ -25,6 +25,21 @@ class ModelConfig(C.Structure):
                 ("tp_rank", C.c_int), ("tp_size", C.c_int)]
 
 
+class LayerSpec(C.Structure):
+    _fields_ = [("mixer", C.c_int), ("heads", C.c_int), ("kv_heads", C.c_int), ("dim", C.c_int), ("vdim", C.c_int),
+                ("window", C.c_int), ("scale", C.c_float), ("qk_norm", C.c_int), ("v_mix", C.c_int), ("mlp", C.c_int),
+                ("experts", C.c_int), ("top", C.c_int), ("expert_ff", C.c_int), ("expert_limit", C.c_float),
+                ("shared_ff", C.c_int), ("shared_limit", C.c_float), ("act_alpha", C.c_float)]
+
+
+class StackConfig(C.Structure):
+    _fields_ = [("width", C.c_int), ("vocab", C.c_int), ("n_layers", C.c_int), ("max_positions", C.c_int),
+                ("norm_eps", C.c_float), ("layers", C.POINTER(LayerSpec))]
+
+
+BF16 = 30
+LAYER_HOOK = C.CFUNCTYPE(None, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int)
+
 _vp, _fp, _ip, _sz = C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t  # device pointers travel as integers
 
 # name -> argtypes; every symbol include/tlhip.h declares (tests/test_capi_symbols.py checks the two agree)
@@ -97,6 +112,14 @@ SIGNATURES = {
     "tl_model_tp_peer_fused": [_vp, _vp],
     "tl_model_graph_nodes": [_vp, _vp],
     "tl_tp_local_group_decode": [_vp, C.c_int, C.c_int, C.c_int, _vp, C.POINTER(C.c_int)],
+    "tl_model_create_stack": [C.POINTER(StackConfig), C.POINTER(C.c_void_p)],
+    "tl_model_set_tensor_named": [_vp, C.c_char_p, C.c_int, C.POINTER(C.c_longlong), C.c_int, _vp],
+    "tl_model_prefill_rows": [_vp, _vp, C.c_int, C.c_int, _vp, C.c_int, _vp],
+    "tl_dense_matmul": [_vp, C.c_int, C.c_int, _fp, _fp, C.c_int, C.c_int, _vp],
+    "tl_swa_attention": [_fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _vp],
+    "tl_resid_rmsnorm": [_fp, _fp, _fp, C.c_int, C.c_int, C.c_float, _vp],
+    "tl_moe_route": [_fp, C.c_int, C.c_int, _vp, _fp, C.c_int, C.c_int, _ip, _fp, _vp],
+    "tl_glu_clamp": [_fp, C.c_int, C.c_int, C.c_float, C.c_float, _fp, _vp],
 }
 
 # include/tlhip_debug.h: measurement / diagnostic hooks (not part of the boundary)
@@ -108,6 +131,7 @@ DEBUG_SIGNATURES = {
     "tl_model_bench_kernel": [_vp, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_double)],
     "tl_chain_set_stamps": [_vp, _sz],
     "tl_debug_gemm_px_launches": [C.POINTER(C.c_longlong)],
+    "tl_model_debug_layer_hook": [_vp, LAYER_HOOK, _vp],
 }
 
 # libtlhip_tools.so (csrc/tl_stream.hip): experiments kept out of the product library; declared in include/tlhip_debug.h

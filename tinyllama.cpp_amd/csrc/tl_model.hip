@@ -19,6 +19,7 @@
 #include <rccl/rccl.h>
 
 #include "tl_internal.h"
+#include "tl_stack.h"
 
 namespace {
 
@@ -40,6 +41,9 @@ struct LayerW {
 
 struct tl_model {
   tl_model_config cfg;
+  // != NULL: a layer-list model (tl_stack.hip) behind this handle instead of the Llama block: it owns weights, caches and the
+  // forward pass; the step state, sampling tail, graph capture and the generation loops below are shared
+  TlStack* stack = nullptr;
   int head_dim = 0, kv_dim = 0;  // kv_dim: LOCAL kv heads x head_dim
   // tensor parallel shard (tp == 1: the whole model): local query heads / kv heads / intermediate columns / vocab rows
   int tp = 1, rank = 0;
@@ -103,6 +107,8 @@ struct tl_model {
     void* planes = nullptr;    // bf16 [3][plane_stride]
     size_t plane_stride = 0;
     float* logits_all = nullptr;  // [cap][vocab], only when all logits were asked for
+    int* rows = nullptr;          // layer-list models: the token rows of a chunk whose logits are wanted
+    int rows_cap = 0;
     int* toks = nullptr;
     int toks_cap = 0;
     // independent GEMMs of a layer (q | k, v and gate | up) run on two streams so that their workgroups share the chip
@@ -225,6 +231,7 @@ extern "C" int tl_model_free(tl_model* m) {
   if (m->graph) hipGraphDestroy(m->graph);
   if (m->graph_exec_sampled) hipGraphExecDestroy(m->graph_exec_sampled);
   if (m->graph_sampled) hipGraphDestroy(m->graph_sampled);
+  tl_stack_free(m->stack);
   hipFree(m->sparams);
   hipFree(m->sample_probs);
   hipFree(m->fattn.sync);
@@ -251,6 +258,7 @@ extern "C" int tl_model_free(tl_model* m) {
   for (float* b : pbufs) hipFree(b);
   hipFree(m->pf.planes);
   hipFree(m->pf.toks);
+  hipFree(m->pf.rows);
   hipFree(m->bt.kv);
   hipFree(m->bt.toks);
   hipFree(m->bt.pos);
@@ -280,6 +288,7 @@ extern "C" int tl_model_set_tensor(tl_model* m, int kind, int layer, int type, c
                                    int cols) {
   TL_REQUIRE(m && host_data, "tl_model_set_tensor: null argument");
   TL_REQUIRE(!m->finalized, "tl_model_set_tensor: model already finalized");
+  TL_REQUIRE(!m->stack, "tl_model_set_tensor: a layer-list model takes its tensors by name (tl_model_set_tensor_named)");
   TL_REQUIRE(rows > 0 && cols > 0, "tl_model_set_tensor: shape %d x %d", rows, cols);
   if (type == TL_BF16) {
     // BF16 tensors (SafeTensors-derived files; weight_management.cpp:888-954 keeps them as uint16 and the CPU forward
@@ -819,6 +828,10 @@ static int chain_check(tl_model* m) {
 
 static int enqueue_step(tl_model* m, StepProf* prof = nullptr, bool sampled = false) {
   hipStream_t s = m->stream;
+  if (m->stack) {  // layer-list model: one token, id and position read from the step state on the device
+    TL_TRY(tl_stack_forward(m->stack, m->state, 1, 0, m->state + 1, nullptr, 1, m->logits, s));
+    return sampled ? enqueue_sample_topk(m, s) : enqueue_sample(m, s);
+  }
   if (m->chain.on && !prof) return enqueue_step_chain(m, sampled);
   PROF_MARK(-1);
   TL_TRY(enqueue_embed(m, s));
@@ -1001,10 +1014,70 @@ static int set_state(tl_model* m, int token, int pos, float penalty, const int* 
   return 0;
 }
 
+extern "C" int tl_model_create_stack(const tl_stack_config* cfg, tl_model** out) {
+  TL_REQUIRE(cfg && out, "tl_model_create_stack: null argument");
+  TlStack* st = nullptr;
+  TL_TRY(tl_stack_create(cfg, &st));
+  tl_model* m = new tl_model();
+  m->stack = st;
+  m->cfg = {};
+  m->cfg.hidden_size = cfg->width;
+  m->cfg.vocab_size = cfg->vocab;
+  m->cfg.num_hidden_layers = cfg->n_layers;
+  m->cfg.max_position_embeddings = cfg->max_positions;
+  m->cfg.rms_norm_eps = cfg->norm_eps;
+  m->cfg.tp_size = 1;
+  hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    tl_stack_free(st);
+    delete m;
+    tl_set_error("tl_model_create_stack: hipStreamCreate failed: %s", hipGetErrorString(e));
+    return 1;
+  }
+  *out = m;
+  return 0;
+}
+
+extern "C" int tl_model_set_tensor_named(tl_model* m, const char* name, int type, const long long* shape, int ndim,
+                                         const void* host_data) {
+  TL_REQUIRE(m && m->stack, "tl_model_set_tensor_named: not a layer-list model (tl_model_set_tensor takes kinds)");
+  return tl_stack_set_tensor(m->stack, name, type, shape, ndim, host_data, m->stream);
+}
+
+// A layer-list model: the engine allocates its caches and workspaces; the step state, logits and arg-max scratch are the
+// same as for the Llama block, and so is the capture of the decode step.
+static int finalize_stack(tl_model* m) {
+  const tl_model_config& c = m->cfg;
+  TL_TRY(tl_stack_finalize(m->stack, m->stream));
+  TL_HIP(hipMalloc(&m->logits, sizeof(float) * (size_t)c.vocab_size));
+  TL_HIP(hipMalloc(&m->cand_v, sizeof(float) * ARGMAX_SLICES));
+  TL_HIP(hipMalloc(&m->cand_i, sizeof(int) * ARGMAX_SLICES));
+  m->hist_cap = c.max_position_embeddings + 64;
+  TL_HIP(hipMalloc(&m->state, sizeof(int) * (kStateHeaderInts + m->hist_cap)));
+  TL_HIP(hipMemsetAsync(m->state, 0, sizeof(int) * (kStateHeaderInts + m->hist_cap), m->stream));
+  m->allocated = true;
+  TL_TRY(set_state(m, 0, 0, 1.0f, nullptr, 0));
+  TL_TRY(enqueue_step(m));  // eager once: validates every launch of the step
+  TL_HIP(hipStreamSynchronize(m->stream));
+  if (const char* e = getenv("TL_NO_GRAPH")) m->no_graph = atoi(e) != 0;
+  if (!m->no_graph) {
+    TL_HIP(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+    const int rc = enqueue_step(m);
+    hipError_t e = hipStreamEndCapture(m->stream, &m->graph);
+    if (rc != 0) return rc;
+    TL_HIP(e);
+    TL_HIP(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
+  }
+  TL_TRY(tl_stack_reset(m->stack, m->stream));  // the warm-up step wrote position 0
+  m->finalized = true;
+  return 0;
+}
+
 extern "C" int tl_model_finalize(tl_model* m) {
   TL_REQUIRE(m, "tl_model_finalize: null handle");
   if (m->finalized) return 0;
   const tl_model_config& c = m->cfg;
+  if (m->stack) return finalize_stack(m);
   TL_REQUIRE(m->tok && m->out && m->out_norm, "tl_model_finalize: token_embd / output / output_norm missing "
              "(the reference has no tied-embedding fallback either, model.cpp:797)");
   m->weight_bytes = gguf_bytes(m->tok, 1) + gguf_bytes(m->out, m->out->rows);
@@ -1102,6 +1175,7 @@ extern "C" int tl_model_finalize(tl_model* m) {
 
 extern "C" int tl_model_reset_kv(tl_model* m) {
   TL_REQUIRE(m && m->finalized, "tl_model_reset_kv: model not finalized");
+  if (m->stack) return tl_stack_reset(m->stack, m->stream);
   TL_HIP(hipMemsetAsync(m->kv_base, 0, sizeof(float) * 2 * m->kv_layer_elems * m->cfg.num_hidden_layers, m->stream));
   TL_HIP(hipStreamSynchronize(m->stream));
   return 0;
@@ -1691,6 +1765,7 @@ static int batch_step(tl_model* m, int T, int* ids_dev, bool advance, float* log
 }
 
 extern "C" int tl_model_batch_init(tl_model* m, int max_batch) {
+  TL_REQUIRE(!m || !m->stack, "tl_model_batch_init: not available for a layer-list model (one sequence, one device)");
   TL_REQUIRE(m && m->finalized, "tl_model_batch_init: model not finalized");
   TL_REQUIRE(m->tp == 1, "tl_model_batch_init: multi-sequence decode is not available on tensor-parallel shards");
   TL_REQUIRE(!m->has_f32, "tl_model_batch_init: a model with F32 / BF16 projection matrices has no multi-sequence step "
@@ -1872,8 +1947,62 @@ extern "C" int tl_model_set_prefill(tl_model* m, int terms, int min_batch) {
   TL_REQUIRE(m, "tl_model_set_prefill: null model");
   TL_REQUIRE(terms == 0 || terms == 1 || terms == 3 || terms == 6, "tl_model_set_prefill: terms must be 0, 1, 3 or 6 (got %d)", terms);
   TL_REQUIRE(min_batch >= 1, "tl_model_set_prefill: min_batch must be >= 1");
+  if (m->stack) TL_TRY(tl_stack_set_terms(m->stack, terms == 0 ? 1 : terms));
   m->prefill_terms = terms;
   m->prefill_min_batch = min_batch;
+  return 0;
+}
+
+// A prompt (or a portion of one) through a layer-list model in chunks; the logits of the listed token rows (ascending;
+// NULL: the last token when n_rows == 1, every token when n_rows == num_tokens) come back as [n_rows][vocab].
+extern "C" int tl_model_prefill_rows(tl_model* m, const int* tokens_host, int num_tokens, int start_pos, const int* rows_host,
+                                     int n_rows, float* logits_host) {
+  TL_REQUIRE(m && m->finalized, "tl_model_prefill_rows: model not finalized");
+  TL_REQUIRE(m->stack, "tl_model_prefill_rows: only layer-list models return chosen rows (use tl_model_prefill)");
+  TL_REQUIRE(tokens_host && num_tokens > 0, "tl_model_prefill_rows: empty prompt");
+  TL_REQUIRE(start_pos >= 0 && start_pos + num_tokens <= m->cfg.max_position_embeddings,
+             "tl_model_prefill_rows: positions [%d,%d) exceed the cache of %d", start_pos, start_pos + num_tokens,
+             m->cfg.max_position_embeddings);
+  TL_REQUIRE(n_rows >= 0 && n_rows <= num_tokens && (n_rows == 0 || logits_host), "tl_model_prefill_rows: bad rows request");
+  TL_REQUIRE(rows_host || n_rows <= 1 || n_rows == num_tokens, "tl_model_prefill_rows: %d rows without a list", n_rows);
+  std::vector<int> rows((size_t)n_rows);
+  for (int i = 0; i < n_rows; ++i) {
+    rows[i] = rows_host ? rows_host[i] : (n_rows == 1 ? num_tokens - 1 : i);
+    TL_REQUIRE(rows[i] >= 0 && rows[i] < num_tokens && (i == 0 || rows[i] > rows[i - 1]),
+               "tl_model_prefill_rows: rows must ascend inside [0, %d)", num_tokens);
+  }
+  const int C = tl_stack_chunk(m->stack);
+  const size_t V = (size_t)m->cfg.vocab_size;
+  TL_TRY(upload_tokens(m, tokens_host, num_tokens, m->stream));
+  if (n_rows > 0 && m->pf.rows_cap < C) {
+    hipFree(m->pf.rows);
+    hipFree(m->pf.logits_all);
+    m->pf.rows = nullptr;
+    m->pf.logits_all = nullptr;
+    TL_HIP(hipMalloc(&m->pf.rows, sizeof(int) * (size_t)C));
+    TL_HIP(hipMalloc(&m->pf.logits_all, sizeof(float) * (size_t)C * V));
+    m->pf.rows_cap = C;
+  }
+  int r0 = 0;
+  for (int t0 = 0; t0 < num_tokens; t0 += C) {
+    const int T = num_tokens - t0 < C ? num_tokens - t0 : C;
+    int r1 = r0;
+    while (r1 < n_rows && rows[r1] < t0 + T) ++r1;
+    std::vector<int> local(rows.begin() + r0, rows.begin() + r1);
+    for (int& r : local) r -= t0;
+    const int nr = r1 - r0;
+    if (nr > 0) {
+      TL_HIP(hipMemcpyAsync(m->pf.rows, local.data(), sizeof(int) * (size_t)nr, hipMemcpyHostToDevice, m->stream));
+      TL_HIP(hipStreamSynchronize(m->stream));  // `local` is this iteration's
+    }
+    TL_TRY(tl_stack_forward(m->stack, m->pf.toks + t0, T, start_pos + t0, nullptr, nr > 0 ? m->pf.rows : nullptr, nr,
+                            m->pf.logits_all, m->stream));
+    if (nr > 0)
+      TL_HIP(hipMemcpyAsync(logits_host + (size_t)r0 * V, m->pf.logits_all, sizeof(float) * (size_t)nr * V,
+                            hipMemcpyDeviceToHost, m->stream));
+    r0 = r1;
+  }
+  TL_HIP(hipStreamSynchronize(m->stream));
   return 0;
 }
 
@@ -1885,6 +2014,13 @@ extern "C" int tl_model_prefill(tl_model* m, const int* tokens_host, int num_tok
   TL_REQUIRE(start_pos >= 0 && start_pos + num_tokens <= m->cfg.max_position_embeddings,
              "tl_model_prefill: positions [%d,%d) exceed max_position_embeddings %d", start_pos, start_pos + num_tokens,
              m->cfg.max_position_embeddings);
+  if (m->stack) {
+    if (all_logits_host) TL_TRY(tl_model_prefill_rows(m, tokens_host, num_tokens, start_pos, nullptr, num_tokens, all_logits_host));
+    else TL_TRY(tl_model_prefill_rows(m, tokens_host, num_tokens, start_pos, nullptr, last_logits_host ? 1 : 0, last_logits_host));
+    if (all_logits_host && last_logits_host)
+      memcpy(last_logits_host, all_logits_host + (size_t)(num_tokens - 1) * m->cfg.vocab_size, sizeof(float) * (size_t)m->cfg.vocab_size);
+    return 0;
+  }
   // (all-token logits of a vocabulary-sharded lm_head are not gathered: that request takes the token-by-token route)
   // (the T x hidden all-reduces of a sharded batched prefill are bandwidth-sized: they stay with RCCL; a group that is
   //  linked by the peer exchange only takes the token-by-token route too)
@@ -1909,6 +2045,7 @@ extern "C" int tl_model_prefill(tl_model* m, const int* tokens_host, int num_tok
 
 extern "C" int tl_model_profile_decode(tl_model* m, int first_token, int start_pos, int n_steps, float* kind_ms_out,
                                        int* kind_launches_out) {
+  TL_REQUIRE(!m || !m->stack, "tl_model_profile_decode: not available for a layer-list model (one sequence, one device)");
   TL_REQUIRE(m && m->finalized && kind_ms_out && kind_launches_out, "tl_model_profile_decode: bad argument");
   TL_REQUIRE(m->tp == 1 || m->linked(), "tl_model_profile_decode: a shard without a communicator cannot step alone");
   TL_REQUIRE(n_steps > 0 && start_pos >= 0 && start_pos + n_steps <= m->cfg.max_position_embeddings,
@@ -1938,8 +2075,23 @@ extern "C" int tl_model_profile_decode(tl_model* m, int first_token, int start_p
   return 0;
 }
 
+extern "C" int tl_model_debug_layer_hook(tl_model* m, tl_layer_hook_fn cb, void* ctx) {
+  TL_REQUIRE(m && m->stack, "tl_model_debug_layer_hook: not a layer-list model");
+  TL_REQUIRE(!cb || m->no_graph || !m->finalized, "tl_model_debug_layer_hook: the decode step is captured (finalize with TL_NO_GRAPH=1)");
+  tl_stack_set_layer_hook(m->stack, cb, ctx);
+  return 0;
+}
+
 extern "C" int tl_model_device_ptr(tl_model* m, int which, int layer, void** dev_out) {
   TL_REQUIRE(m && m->finalized && dev_out, "tl_model_device_ptr: bad argument");
+  if (m->stack) {
+    if (which == 2) {
+      *dev_out = const_cast<float*>(tl_stack_residual(m->stack));
+      return 0;
+    }
+    TL_REQUIRE(which == 0 || which == 1, "tl_model_device_ptr: unknown buffer %d", which);
+    return tl_stack_cache_ptr(m->stack, which, layer, dev_out);
+  }
   if (which == 2) {
     *dev_out = m->x;
     return 0;
@@ -1958,6 +2110,10 @@ extern "C" int tl_model_prefill_planes_bytes(const tl_model* m, size_t* bytes_ou
 
 extern "C" int tl_model_bytes_per_token(const tl_model* m, int pos, double* weight_bytes, double* kv_bytes) {
   TL_REQUIRE(m && m->finalized, "tl_model_bytes_per_token: model not finalized");
+  if (m->stack) {
+    tl_stack_bytes_per_token(m->stack, pos, weight_bytes, kv_bytes);
+    return 0;
+  }
   if (weight_bytes) *weight_bytes = m->weight_bytes;
   if (kv_bytes)  // read K and V of positions 0..pos, write one position
     *kv_bytes = (double)m->cfg.num_hidden_layers * 2.0 * ((double)pos + 2.0) * m->kv_dim * sizeof(float);
@@ -1989,6 +2145,7 @@ extern "C" int tl_tp_unique_id(void* id_out_128) {
   return 0;
 }
 extern "C" int tl_model_tp_init(tl_model* m, const void* unique_id_128) {
+  TL_REQUIRE(!m || !m->stack, "tl_model_tp_init: not available for a layer-list model (one sequence, one device)");
   TL_REQUIRE(m && unique_id_128, "tl_model_tp_init: null argument");
   TL_REQUIRE(!m->finalized, "tl_model_tp_init: call before tl_model_finalize (the decode graph captures the collectives)");
   // tp_size 1 needs no communicator; TL_TP_SELFTEST=1 makes a one-rank communicator anyway, so that the RCCL calls and
@@ -2004,6 +2161,7 @@ extern "C" int tl_model_tp_init(tl_model* m, const void* unique_id_128) {
 
 // ---- peer-to-peer exchange wiring (tl_peer.hip) ------------------------------------------------------------------------
 extern "C" int tl_model_tp_peer_export(tl_model* m, void* handle_out_64) {
+  TL_REQUIRE(!m || !m->stack, "tl_model_tp_peer_export: not available for a layer-list model (one sequence, one device)");
   TL_REQUIRE(m && handle_out_64, "tl_model_tp_peer_export: null argument");
   TL_REQUIRE(!m->finalized, "tl_model_tp_peer_export: call before tl_model_finalize (the decode graph captures the exchanges)");
   TL_REQUIRE(m->tp >= 2 && m->tp <= TL_PEER_MAX_RANKS, "tl_model_tp_peer_export: tp_size %d outside 2..%d", m->tp,

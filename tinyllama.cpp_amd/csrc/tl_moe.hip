@@ -1,0 +1,225 @@
+// tl_moe.hip — mixture-of-experts feed-forward: router, grouping plan, the experts' clamped gated activation, and the
+// one-token (decode) form of the experts.
+//
+//   router   logits z = W_r x + b in FP32 (bf16 weights widened exactly); the `top` largest are chosen (equal logits: the
+//            lower index first) and weighted by the softmax over the chosen logits only.
+//   plan     the T * top (token, choice) slots grouped by expert: off[e] .. off[e + 1] index slot_of[]. The order inside a
+//            group is whatever the atomics give; no result depends on it (every slot's output is computed on its own and
+//            summed per token in choice order).
+//   act      y = g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).
+//   decode   one token: gate/up GEMVs of the chosen experts (+ the shared expert) with the activation applied in the same
+//            launch, then one launch in which a wave owns an output row and sums the chosen experts' down rows with the
+//            router weights (and the shared expert's with weight 1).
+#include <math.h>
+
+#include "tl_stack.h"
+
+namespace {
+
+constexpr int kMaxExperts = 1024;
+
+__device__ __forceinline__ float bf2f(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+
+// dot of a bf16 row with an FP32 vector over the lanes of a wave; result in every lane
+__device__ __forceinline__ float wave_dot(const unsigned short* __restrict__ wr, const float* __restrict__ x, int n, bool vec,
+                                          int lane) {
+  float s = 0.0f;
+  if (vec) {
+    for (int k = lane * 8; k < n; k += 512) {
+      const uint4 w4 = *reinterpret_cast<const uint4*>(wr + k);
+      const float4 x0 = *reinterpret_cast<const float4*>(x + k);
+      const float4 x1 = *reinterpret_cast<const float4*>(x + k + 4);
+      s += __uint_as_float(w4.x << 16) * x0.x + __uint_as_float(w4.x & 0xffff0000u) * x0.y +
+           __uint_as_float(w4.y << 16) * x0.z + __uint_as_float(w4.y & 0xffff0000u) * x0.w +
+           __uint_as_float(w4.z << 16) * x1.x + __uint_as_float(w4.z & 0xffff0000u) * x1.y +
+           __uint_as_float(w4.w << 16) * x1.z + __uint_as_float(w4.w & 0xffff0000u) * x1.w;
+    }
+  } else {
+    for (int k = lane; k < n; k += 64) s += bf2f(wr[k]) * x[k];
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
+  return s;
+}
+
+__global__ __launch_bounds__(256) void router_kernel(const RouterArgs a, int vec) {
+  extern __shared__ float z[];  // [experts]
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float* x = a.x + (size_t)t * a.width;
+  for (int e = wave; e < a.experts; e += 4) {
+    const float s = wave_dot(a.w + (size_t)e * a.width, x, a.width, vec != 0, lane);
+    if (lane == 0) z[e] = s + (a.b ? a.b[e] : 0.0f);
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // `top` rounds: the lanes scan the experts not yet chosen for the largest logit (lower index wins among equals)
+    float mx = 0.0f, denom = 0.0f, mine = 0.0f;
+    int my_id = -1;
+    for (int j = 0; j < a.top; ++j) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int e = lane; e < a.experts; e += 64) {
+        const float v = z[e];
+        if (v > bv || (v == bv && e < bi)) {
+          bv = v;
+          bi = e;
+        }
+      }
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(bv, o);
+        const int oi = __shfl_xor(bi, o);
+        if (ov > bv || (ov == bv && oi < bi)) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (bi == 0x7fffffff) bi = 0;  // only when every logit is NaN
+      if (j == 0) mx = bv;
+      const float p = expf(bv - mx);
+      denom += p;
+      if (lane == j % 64 && j < 64) {
+        mine = p;
+        my_id = bi;
+      }
+      if (j >= 64 && lane == 0) {  // more than 64 choices: written unnormalised, fixed up below
+        a.ids[t * a.top + j] = bi;
+        a.wts[t * a.top + j] = p;
+      }
+      if (lane == 0) z[bi] = -INFINITY;  // chosen: out of the next rounds
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if (lane < a.top && lane < 64) {
+      a.ids[t * a.top + lane] = my_id;
+      a.wts[t * a.top + lane] = mine / denom;
+    }
+    if (a.top > 64 && lane == 0)
+      for (int j = 64; j < a.top; ++j) a.wts[t * a.top + j] /= denom;
+  }
+}
+
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ ids, int n_slots, int experts,
+                                                        int* __restrict__ off, int* __restrict__ slot_of) {
+  __shared__ int cnt[kMaxExperts + 1];
+  for (int e = threadIdx.x; e <= experts; e += 1024) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_slots; i += 1024) atomicAdd(&cnt[ids[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int e = 0; e < experts; ++e) {
+      const int c = cnt[e];
+      off[e] = run;
+      cnt[e] = run;  // becomes the group's cursor
+      run += c;
+    }
+    off[experts] = run;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n_slots; i += 1024) slot_of[atomicAdd(&cnt[ids[i]], 1)] = i;
+}
+
+__device__ __forceinline__ float glu_act(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+}
+
+__global__ __launch_bounds__(256) void glu_act_kernel(const float* __restrict__ in, size_t n, int ff, float limit, float alpha,
+                                                      float* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const size_t p = i / ff;
+  const int c = (int)(i - p * ff);
+  out[i] = glu_act(in[p * 2 * ff + c], in[p * 2 * ff + ff + c], limit, alpha);
+}
+
+// grid: (rows of 4 waves over max(ff, sff), top + 1). Slot j < top: expert ids[j]; slot top: the shared expert.
+__global__ __launch_bounds__(256) void moe_decode_gu_kernel(const MoeDecodeArgs a, int vec) {
+  const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6), j = blockIdx.y;
+  const bool shared = j == a.top;
+  const int ff = shared ? a.sff : a.ff;
+  if (r >= ff) return;
+  const unsigned short* gu = shared ? a.sgu : a.gu + (size_t)a.ids[j] * 2 * a.ff * a.width;
+  const float g = wave_dot(gu + (size_t)r * a.width, a.x, a.width, vec != 0, lane);
+  const float u = wave_dot(gu + (size_t)(ff + r) * a.width, a.x, a.width, vec != 0, lane);
+  if (lane == 0) a.act[(size_t)j * a.ff + r] = glu_act(g, u, shared ? a.slimit : a.limit, a.alpha);
+}
+
+__global__ __launch_bounds__(256) void moe_decode_down_kernel(const MoeDecodeArgs a, int vec_e, int vec_s) {
+  const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= a.width) return;
+  float y = 0.0f;
+  for (int j = 0; j < a.top; ++j) {
+    const unsigned short* d = a.down + ((size_t)a.ids[j] * a.width + r) * a.ff;
+    y += a.wts[j] * wave_dot(d, a.act + (size_t)j * a.ff, a.ff, vec_e != 0, lane);
+  }
+  if (a.sdown) y += wave_dot(a.sdown + (size_t)r * a.sff, a.act + (size_t)a.top * a.ff, a.sff, vec_s != 0, lane);
+  if (lane == 0) a.y[r] = y;
+}
+
+}  // namespace
+
+int tl_launch_router(const RouterArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.x && a.w && a.ids && a.wts && a.T > 0 && a.width > 0, "router: bad arguments");
+  TL_REQUIRE(a.experts > 0 && a.experts <= kMaxExperts, "router: %d experts outside (0, %d]", a.experts, kMaxExperts);
+  TL_REQUIRE(a.top > 0 && a.top <= a.experts, "router: top %d of %d experts", a.top, a.experts);
+  const int vec = (a.width & 7) == 0 && ((size_t)a.x & 15) == 0 && ((size_t)a.w & 15) == 0;
+  router_kernel<<<a.T, 256, sizeof(float) * a.experts, s>>>(a, vec);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_moe_plan(const int* ids, int n_slots, int experts, int* off, int* slot_of, hipStream_t s) {
+  TL_REQUIRE(ids && off && slot_of && n_slots > 0, "moe_plan: bad arguments");
+  TL_REQUIRE(experts > 0 && experts <= kMaxExperts, "moe_plan: %d experts outside (0, %d]", experts, kMaxExperts);
+  moe_plan_kernel<<<1, 1024, 0, s>>>(ids, n_slots, experts, off, slot_of);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_glu_act(const float* in, int P, int ff, float limit, float alpha, float* out, hipStream_t s) {
+  TL_REQUIRE(in && out && P > 0 && ff > 0, "glu_act: bad arguments");
+  const size_t n = (size_t)P * ff;
+  glu_act_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(in, n, ff, limit, alpha, out);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_moe_decode(const MoeDecodeArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.x && a.ids && a.wts && a.gu && a.down && a.act && a.y && a.width > 0 && a.ff > 0 && a.top > 0,
+             "moe_decode: bad arguments");
+  TL_REQUIRE(!a.sgu == !a.sdown && (!a.sgu || a.sff > 0), "moe_decode: shared expert half given");
+  const bool al = ((size_t)a.x & 15) == 0 && ((size_t)a.act & 15) == 0 && ((size_t)a.gu & 15) == 0 && ((size_t)a.down & 15) == 0 &&
+                  ((size_t)a.sgu & 15) == 0 && ((size_t)a.sdown & 15) == 0;
+  const int vec_x = al && (a.width & 7) == 0;
+  // the activations of slot j start at act + j * ff: 16-byte pieces need ff % 8 == 0 (which also aligns the rows of `down`)
+  const int vec_e = al && (a.ff & 7) == 0;
+  const int vec_s = vec_e && (a.sff & 7) == 0;
+  const int ffmax = a.sgu && a.sff > a.ff ? a.sff : a.ff;
+  moe_decode_gu_kernel<<<dim3((ffmax + 3) / 4, a.top + (a.sgu ? 1 : 0)), 256, 0, s>>>(a, vec_x);
+  moe_decode_down_kernel<<<(a.width + 3) / 4, 256, 0, s>>>(a, vec_e, vec_s);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int tl_moe_route(const float* x_dev, int num_tokens, int width, const void* w_bf16_dev, const float* bias_dev,
+                            int experts, int top, int* ids_dev, float* weights_dev, void* stream) {
+  RouterArgs a = {};
+  a.x = x_dev;
+  a.T = num_tokens;
+  a.width = width;
+  a.experts = experts;
+  a.top = top;
+  a.w = static_cast<const uint16_t*>(w_bf16_dev);
+  a.b = bias_dev;
+  a.ids = ids_dev;
+  a.wts = weights_dev;
+  return tl_launch_router(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_glu_clamp(const float* gate_up_dev, int rows, int ff, float limit, float alpha, float* out_dev, void* stream) {
+  return tl_launch_glu_act(gate_up_dev, rows, ff, limit, alpha, out_dev, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,139 @@
+// tl_stack.h — inside libtlhip.so: the layer-list engine (tl_stack.hip) and the operators it is built from. A "stack" model
+// is described layer by layer (tl_stack_config, include/tlhip.h) instead of by the fixed Llama block of tl_model.hip; it
+// lives behind the same tl_model handle and entry points (decode step, prefill, generation, cache reset).
+//
+// Operators (each with its sizes and constants as arguments, so that another design can use them):
+//   tl_dense.hip  bf16 weight matrices [rows][cols]: GEMV (one token) and MFMA GEMM (a chunk of tokens, optionally grouped
+//                 by expert with gathered input rows / scattered output rows); FP32 activations and accumulation
+//   tl_swa.hip    sliding-window attention without rotation, key and value sizes independent, over a flat FP32 cache
+//   tl_moe.hip    router (top-k, softmax over the chosen logits), grouping plan, clamped gated activation, decode GEMVs
+//   tl_norm.hip   RMS norms with zero-centred weights: embedding gather + norm, whole-projection q/k norm + value mixing +
+//                 cache write, residual += norm(sublayer output), row-gathering norm in front of the head
+#pragma once
+#include "tl_internal.h"
+
+// ---- tl_dense.hip ------------------------------------------------------------------------------------------------------
+struct DenseArgs {
+  const uint16_t* w;     // bf16 [groups][rows][cols], row-major (as the checkpoint stores it: y = W x)
+  int rows, cols;        // output features, input features
+  const float* x;        // activations, row r at x + r * ldx
+  int ldx;
+  float* y;              // outputs, row r at y + r * ldy
+  int ldy;
+  int T;                 // items (tokens); with group_off: upper bound of the items of one group
+  int terms;             // bf16 MFMAs per product: 1 = activations rounded to bf16, 3 = FP32-grade (hi + mid + lo split)
+  const int* x_rows;     // optional (device): item i reads activation row x_rows[i] / x_div
+  int x_div;
+  const int* y_rows;     // optional (device): item i writes output row y_rows[i]
+  int groups;            // > 1 (or group_off set): group g uses matrix g and the items [group_off[g], group_off[g+1])
+  const int* group_off;  // device, groups + 1 entries
+};
+int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s);
+// y[rows] = W x for one token, FP32 throughout (weights widened exactly)
+int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s);
+
+// ---- tl_swa.hip --------------------------------------------------------------------------------------------------------
+struct SwaArgs {
+  const float* q;   // [T][ldq]: head h of token t at q + t * ldq + h * dim
+  int ldq;
+  const float* kc;  // keys   [max_pos][kv_heads * dim]
+  const float* vc;  // values [max_pos][kv_heads * vdim]
+  float* out;       // [T][heads * vdim]
+  int T, heads, kv_heads, dim, vdim;
+  int window;       // position i sees j with 0 <= i - j < window (<= 0: every j <= i)
+  float scale;
+  int start_pos;    // position of token 0 ...
+  const int* pos_dev;  // ... or, when set, read from the device (graph replay)
+};
+int tl_launch_swa(const SwaArgs& a, hipStream_t s);
+
+// ---- tl_norm.hip -------------------------------------------------------------------------------------------------------
+// x[t] = embed[token[t]] / rms * (1 + w)   (bf16 table; an id outside the table embeds as zeros)
+int tl_launch_embed_norm(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, const float* w, float eps,
+                         float* x, hipStream_t s);
+struct QkvPostArgs {
+  float* qkv;            // [T][ld]: q (qd) | k (kd) | v (vd) of a token; q is normalised in place
+  int ld, qd, kd, vd;
+  const float* q_norm;   // plain weights over the whole projection (NULL: no norm)
+  const float* k_norm;
+  float eps;
+  float* kc;             // [max_pos][kd], row pos
+  float* vc;             // [max_pos][vd]
+  int T, start_pos;
+  const int* pos_dev;
+  int vmix;              // 0: v as it is; 1: this layer's v is kept in v_first; 2: v = (1 - lambda) v + lambda v_first
+  float* v_first;        // [T][vd]
+  const float* lambda;   // device scalar (vmix == 2)
+};
+int tl_launch_qkv_post(const QkvPostArgs& a, hipStream_t s);
+struct ResidNormArgs {
+  float* x;              // [T][width] residual stream, updated in place: x += y / rms(y) * (1 + w)
+  int T, width;
+  const float* a;        // optional [T][width]
+  const float* slots;    // optional [T * top][width] expert outputs, weighted by slot_w
+  const float* slot_w;   // [T * top]
+  int top;
+  const float* w;
+  float eps;
+};
+int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s);
+// out[i] = x[rows[i]] / rms * (1 + w)   (rows == NULL: row i)
+int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, const float* w, float eps, float* out,
+                        hipStream_t s);
+
+// ---- tl_moe.hip --------------------------------------------------------------------------------------------------------
+struct RouterArgs {
+  const float* x;        // [T][width]
+  int T, width, experts, top;
+  const uint16_t* w;     // bf16 [experts][width]
+  const float* b;        // [experts]
+  int* ids;              // [T][top] chosen experts, largest logit first
+  float* wts;            // [T][top] softmax over the chosen logits
+};
+int tl_launch_router(const RouterArgs& a, hipStream_t s);
+// slots (t * top + j) grouped by expert: off[experts + 1], slot_of[T * top]
+int tl_launch_moe_plan(const int* ids, int n_slots, int experts, int* off, int* slot_of, hipStream_t s);
+// out[p][i] = g * sigmoid(alpha * g) * (u + 1), g = min(in[p][i], limit), u = clamp(in[p][ff + i], -limit, limit)
+int tl_launch_glu_act(const float* in, int P, int ff, float limit, float alpha, float* out, hipStream_t s);
+// one token: the chosen experts' (and the shared expert's) gate/up GEMVs + activation, then the down GEMVs summed with the
+// router weights into y[width]. gu matrices are [2 * ff][width] (gate rows, then up rows), down [width][ff].
+struct MoeDecodeArgs {
+  const float* x;        // [width]
+  int width, top;
+  const int* ids;        // [top] (device)
+  const float* wts;      // [top]
+  const uint16_t* gu;    // [experts][2 * ff][width]
+  const uint16_t* down;  // [experts][width][ff]
+  int ff;
+  float limit;
+  const uint16_t* sgu;   // shared expert (NULL: none)
+  const uint16_t* sdown;
+  int sff;
+  float slimit;
+  float alpha;
+  float* act;            // scratch [top * ff + sff]
+  float* y;              // [width]
+};
+int tl_launch_moe_decode(const MoeDecodeArgs& a, hipStream_t s);
+
+// ---- tl_stack.hip: the engine ------------------------------------------------------------------------------------------
+struct TlStack;
+int tl_stack_create(const tl_stack_config* cfg, TlStack** out);
+void tl_stack_free(TlStack* st);
+int tl_stack_set_tensor(TlStack* st, const char* name, int dtype, const long long* shape, int ndim, const void* host_data,
+                        hipStream_t s);
+int tl_stack_finalize(TlStack* st, hipStream_t s);
+int tl_stack_reset(TlStack* st, hipStream_t s);
+int tl_stack_set_terms(TlStack* st, int terms);
+// T tokens (ids on the device) at positions start_pos.. (or *pos_dev..): updates the caches; logits of the n_rows token rows
+// listed in rows_dev (NULL with n_rows == 1: the last token) go to logits_dev [n_rows][vocab]. T <= tl_stack_chunk().
+int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, const int* pos_dev, const int* rows_dev,
+                     int n_rows, float* logits_dev, hipStream_t s);
+int tl_stack_chunk(const TlStack* st);
+int tl_stack_cache_ptr(TlStack* st, int which, int layer, void** out);
+// residual stream of the last forward call, [T][width] (tests)
+const float* tl_stack_residual(const TlStack* st);
+void tl_stack_bytes_per_token(const TlStack* st, int pos, double* weight_bytes, double* kv_bytes);
+// called after every layer of a forward call when set (tests: the residual stream layer by layer)
+typedef void (*tl_stack_layer_hook)(void* ctx, int layer, const float* x_dev, int T, int width);
+void tl_stack_set_layer_hook(TlStack* st, tl_stack_layer_hook hook, void* ctx);

@@ -432,3 +432,93 @@ class Model:
             self.free()
         except Exception:
             pass
+
+
+def stack_config_struct(config, max_pos):
+    """The ctypes form (tl_stack_config) of a layer-list configuration given as config.json's dictionary; returns
+    (struct, the array it points into). The C++ host does the same from the file (host/tl_stack_config.cpp); this one
+    serves tests and benches that build models in memory."""
+    layers = config["layers"]
+    arr = (capi.LayerSpec * len(layers))()
+    for i, L in enumerate(layers):
+        if L["type"] != "attention":
+            raise ValueError(f"layer {i}: unknown type {L['type']!r}")
+        mx, ml, sp = L["mixer"], L.get("mlp"), arr[i]
+        sp.mixer, sp.heads, sp.kv_heads, sp.dim, sp.vdim = 0, mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+        sp.window = int((mx.get("mask") or {}).get("size", 0))
+        sp.scale, sp.qk_norm, sp.v_mix = float(mx["scale"]), 1, int(bool(mx.get("v_mix")))
+        sp.act_alpha = 1.702
+        if ml is not None:
+            if ml.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {ml.get('kind')!r}")
+            sp.mlp, sp.experts, sp.top = 1, ml["router"]["experts"], ml["router"]["top"]
+            sp.expert_ff, sp.expert_limit = ml["expert"]["ff"], float(ml["expert"]["limit"])
+            sh = ml.get("shared")
+            if sh:
+                sp.shared_ff, sp.shared_limit = sh["ff"], float(sh["limit"])
+    c = capi.StackConfig(config["width"], config["vocab"], len(layers), int(max_pos), float(config["norm"]["eps"]), arr)
+    return c, arr
+
+
+class StackModel(Model):
+    """A layer-list model (tl_model_create_stack) behind the same handle and methods as Model. `config` is config.json's
+    dictionary; tensors come by checkpoint name as uint16 arrays holding bf16 bits (or float32 arrays for vectors)."""
+
+    def __init__(self, config, max_pos=2048):
+        _ensure_init()
+        self.config = config
+        self.cfg = {"vocab": config["vocab"], "hidden": config["width"], "n_layers": len(config["layers"]), "max_pos": max_pos}
+        self.tp_rank, self.tp_size = 0, 1
+        c, self._keep = stack_config_struct(config, max_pos)
+        h = C.c_void_p()
+        check(lib().tl_model_create_stack(C.byref(c), C.byref(h)), "tl_model_create_stack")
+        self.h = h.value
+        self._hook = None
+
+    def set_tensor(self, name, arr):
+        arr = np.ascontiguousarray(arr)
+        typ = {np.dtype(np.uint16): capi.BF16, np.dtype(np.float32): capi.F32}[arr.dtype]
+        shape = (C.c_longlong * max(arr.ndim, 1))(*arr.shape)
+        check(lib().tl_model_set_tensor_named(self.h, name.encode(), typ, shape, arr.ndim, arr.ctypes.data),
+              f"tl_model_set_tensor_named({name})")
+
+    def load(self, tensors):
+        for name, arr in tensors.items():
+            self.set_tensor(name, arr)
+        self.finalize()
+        return self
+
+    def prefill_rows(self, tokens, start_pos=0, rows=None):
+        """A prompt portion at positions start_pos..; logits [len(rows), vocab] of the listed token rows (None: all)."""
+        toks = np.ascontiguousarray(tokens, np.int32)
+        rows = np.arange(toks.size, dtype=np.int32) if rows is None else np.ascontiguousarray(rows, np.int32)
+        out = np.empty((rows.size, self.cfg["vocab"]), np.float32)
+        check(lib().tl_model_prefill_rows(self.h, toks.ctypes.data, toks.size, int(start_pos), rows.ctypes.data, rows.size,
+                                          out.ctypes.data), "tl_model_prefill_rows")
+        return out
+
+    def capture_layers(self, fn):
+        """Run fn() with the layer hook set; returns [(layer, residual [T, width])] in call order."""
+        got = []
+
+        def cb(_ctx, layer, x_dev, T, width):
+            a = np.empty((T, width), np.float32)
+            check(lib().tl_memcpy_d2h(a.ctypes.data, x_dev, a.nbytes, None), "d2h")
+            got.append((layer, a))
+
+        self._hook = capi.LAYER_HOOK(cb)
+        check(lib().tl_model_debug_layer_hook(self.h, self._hook, None), "tl_model_debug_layer_hook")
+        try:
+            fn()
+        finally:
+            check(lib().tl_model_debug_layer_hook(self.h, capi.LAYER_HOOK(0), None), "tl_model_debug_layer_hook")
+        return got
+
+    def kv_cache(self, layer, n_pos):
+        mx = self.config["layers"][layer]["mixer"]
+        out = []
+        for which, d in ((0, mx["kv_heads"] * mx["dim"]), (1, mx["kv_heads"] * mx["vdim"])):
+            a = np.empty((n_pos, d), np.float32)
+            check(lib().tl_memcpy_d2h(a.ctypes.data, self.device_ptr(which, layer), a.nbytes, None), "d2h")
+            out.append(a)
+        return out

@@ -255,3 +255,104 @@ def write_gguf(path, cfg, tensors, alignment=32, extra_kvs=()):
         if f.tell() < end:
             f.write(b"\0" * (end - f.tell()))
     return path
+
+
+# ---- layer-list models (tl_model_create_stack): random-init checkpoints in their on-disk form (config.json + safetensors) ----
+def to_bf16(a):
+    """float32 array -> uint16 array of its bf16 bits (round to nearest even)."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+
+def from_bf16(b):
+    return (np.asarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def stack_layer(heads, kv_heads, dim, vdim, window, v_mix=True, experts=4, top=2, ff=32, shared_ff=64, limit=1.0,
+                shared_limit=1.0, scale=None, mlp=True):
+    """One entry of config.json's "layers" list. window None: no mask entry (every earlier position is seen)."""
+    mixer = {"dim": dim, "heads": heads, "kv_heads": kv_heads, "scale": float(scale if scale is not None else dim ** -0.5),
+             "v_mix": bool(v_mix), "vdim": vdim}
+    if window is not None:
+        mixer["mask"] = {"size": int(window)}
+    ml = None
+    if mlp:
+        ml = {"kind": "moe", "expert": {"ff": ff, "limit": float(limit)}, "router": {"experts": experts, "top": top},
+              "shared": {"ff": shared_ff, "limit": float(shared_limit)} if shared_ff else None}
+    return {"type": "attention", "mixer": mixer, "mlp": ml}
+
+
+def stack_config(width, vocab, layers, eps=1e-5):
+    return {"architecture": "Ralasun", "layers": list(layers), "norm": {"eps": float(eps)}, "vocab": int(vocab),
+            "width": int(width)}
+
+
+def build_stack(config, seed=0, gain=1.0):
+    """Random tensors {checkpoint name: uint16 bf16 bits}. Projections have std gain / sqrt(fan_in); norm weights are small
+    values around zero (the norms apply 1 + w), query/key norm weights around one, router biases of the size of the logits'
+    spread, mixing coefficients in (0.2, 0.8)."""
+    rng = np.random.default_rng(seed)
+    W, V = config["width"], config["vocab"]
+    t = {}
+
+    def mat(name, rows, cols, std=None):
+        t[name] = to_bf16(rng.standard_normal((rows, cols)).astype(np.float32) * (std or gain / np.sqrt(cols)))
+
+    def vec(name, n, centre, spread):
+        t[name] = to_bf16((centre + spread * rng.standard_normal(n)).astype(np.float32))
+
+    mat("embed", V, W, 1.0)
+    vec("embed.norm", W, 0.0, 0.1)
+    vec("final.norm", W, 0.0, 0.1)
+    mat("head", V, W)
+    for i, L in enumerate(config["layers"]):
+        mx, ml, p = L["mixer"], L.get("mlp"), f"l{i}."
+        H, G, d, dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+        vec(p + "norm1", W, 0.0, 0.1)
+        mat(p + "mix.q", H * d, W)
+        mat(p + "mix.k", G * d, W)
+        mat(p + "mix.v", G * dv, W)
+        mat(p + "mix.o", W, H * dv)
+        vec(p + "mix.q.norm", H * d, 1.0, 0.2)
+        vec(p + "mix.k.norm", G * d, 1.0, 0.2)
+        if mx.get("v_mix"):
+            t[p + "mix.vmix"] = to_bf16(np.array(rng.uniform(0.2, 0.8), np.float32))
+        if ml is not None:
+            vec(p + "norm2", W, 0.0, 0.1)
+            E, ff = ml["router"]["experts"], ml["expert"]["ff"]
+            mat(p + "mlp.router", E, W)
+            vec(p + "mlp.router.b", E, 0.0, 0.5)
+            for e in range(E):
+                mat(p + f"mlp.e{e}.gate", ff, W, 2.0 / np.sqrt(W))
+                mat(p + f"mlp.e{e}.up", ff, W, 2.0 / np.sqrt(W))
+                mat(p + f"mlp.e{e}.down", W, ff)
+            if ml.get("shared"):
+                sff = ml["shared"]["ff"]
+                mat(p + "mlp.shared.gate", sff, W, 2.0 / np.sqrt(W))
+                mat(p + "mlp.shared.up", sff, W, 2.0 / np.sqrt(W))
+                mat(p + "mlp.shared.down", W, sff)
+    return t
+
+
+def write_stack_dir(path, config, tensors):
+    """config.json + model.safetensors (8-byte little-endian header length, JSON header, data) under `path`."""
+    import json
+    import os
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(config, f, indent=1)
+    header, off, blobs = {}, 0, []
+    for name, a in tensors.items():
+        a = np.ascontiguousarray(a)
+        dt = {np.dtype(np.uint16): "BF16", np.dtype(np.float32): "F32", np.dtype(np.int32): "I32"}[a.dtype]
+        b = a.tobytes()
+        header[name] = {"dtype": dt, "shape": list(a.shape), "data_offsets": [off, off + len(b)]}
+        off += len(b)
+        blobs.append(b)
+    h = json.dumps(header, separators=(",", ":")).encode()
+    h += b" " * (-len(h) % 8)
+    with open(os.path.join(path, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(h)))
+        f.write(h)
+        for b in blobs:
+            f.write(b)
