@@ -33,7 +33,8 @@ int tlh_gguf_model_config(const tlh_gguf* g, int out[9], float eps_theta[2]);
 
 /* ---- session : TinyLlamaSession (api.h:42-78) on token ids ---- */
 typedef struct tlh_session tlh_session;
-int tlh_session_open(const char* gguf_path, int device, int max_context, tlh_session** out);
+/* path: a .gguf file, or a checkpoint folder (config.json + model.safetensors); the family is chosen by the architecture named there */
+int tlh_session_open(const char* path, int device, int max_context, tlh_session** out);
 int tlh_session_close(tlh_session* s);
 int tlh_session_set_repetition_penalty(tlh_session* s, float penalty);
 int tlh_session_seed(tlh_session* s, uint32_t seed);
@@ -47,6 +48,16 @@ int tlh_session_set_max_batch(tlh_session* s, int max_batch_size);
  * empty prompt list, more prompts than max_batch_size. */
 int tlh_session_generate_batch(tlh_session* s, const int* prompt_ids, const int* offsets, int n_prompts, int steps,
                                float temperature, int top_k, float top_p, int* out_ids, int* out_lens);
+/* Session::forward: the step function for callers that schedule themselves. Feeds n_tokens ids at positions start_pos.. on
+ * top of what earlier calls left in the cache; logits_out[n_want][vocab] = the logits of the token rows want[] (ascending).
+ * One token at a position > 0 runs the decode step, anything else the batched prefill. tlh_session_reset gives the cache
+ * back; tlh_session_set_exact(1) makes the prompt-chunk matrix products FP32-grade (0: the family's serving default). */
+int tlh_session_forward(tlh_session* s, const int* tokens, int n_tokens, int start_pos, const int* want, int n_want,
+                        float* logits_out);
+int tlh_session_reset(tlh_session* s);
+int tlh_session_set_exact(tlh_session* s, int on);
+/* out[0..3] = vocabulary, width, layers, cache rows; the architecture name the checkpoint carries into arch_buf */
+int tlh_session_info(const tlh_session* s, int out[4], char* arch_buf, size_t buf_len);
 /* load statistics: tensors uploaded, quantized bytes taken from the mapping, seconds for open() */
 int tlh_session_load_stats(const tlh_session* s, uint64_t* tensors, uint64_t* quantized_bytes, double* seconds);
 

@@ -7,6 +7,9 @@
 #include "tl_session.hpp"
 #include "tlhost.h"
 
+#include <algorithm>
+#include <cstdio>
+
 namespace {
 thread_local std::string g_err;
 template <typename F>
@@ -179,6 +182,34 @@ int tlh_session_generate_batch(tlh_session* s, const int* prompt_ids, const int*
       if (n > 0) memcpy(out_ids + (size_t)i * steps, out[i].data(), sizeof(int) * (size_t)n);
     }
   });
+}
+int tlh_session_forward(tlh_session* s, const int* tokens, int n_tokens, int start_pos, const int* want, int n_want,
+                        float* logits_out) {
+  if (!s || !tokens || n_tokens <= 0 || n_want < 0 || (n_want > 0 && (!want || !logits_out)))
+    return fail("tlh_session_forward: bad argument");
+  return guarded([&] {
+    const std::vector<float> l = s->s->forward(std::vector<int>(tokens, tokens + n_tokens), start_pos,
+                                               std::vector<int>(want, want + n_want));
+    std::copy(l.begin(), l.end(), logits_out);
+  });
+}
+int tlh_session_reset(tlh_session* s) {
+  if (!s) return fail("tlh_session_reset: null handle");
+  return guarded([&] { s->s->reset(); });
+}
+int tlh_session_set_exact(tlh_session* s, int on) {
+  if (!s) return fail("tlh_session_set_exact: null handle");
+  return guarded([&] { s->s->set_exact(on != 0); });
+}
+int tlh_session_info(const tlh_session* s, int out[4], char* arch_buf, size_t buf_len) {
+  if (!s || !out) return fail("tlh_session_info: bad argument");
+  const tlhost::ModelConfig& c = s->s->get_config();
+  out[0] = c.vocab_size;
+  out[1] = c.hidden_size;
+  out[2] = c.num_hidden_layers;
+  out[3] = c.max_position_embeddings;
+  if (arch_buf && buf_len) snprintf(arch_buf, buf_len, "%s", c.architecture.c_str());
+  return 0;
 }
 int tlh_session_load_stats(const tlh_session* s, uint64_t* tensors, uint64_t* qbytes, double* seconds) {
   if (!s) return fail("tlh_session_load_stats: null handle");

@@ -1,7 +1,9 @@
 // tl_run — minimal command-line driver of the C++ host layer (the reference's main.cpp drives TinyLlamaSession).
-//   tl_run model.gguf --ids 1,15,27 [--steps 32] [--temperature 0] [--top-k 40] [--top-p 0.9] [--penalty 1.3]
+//   tl_run MODEL --ids 1,15,27 [--steps 32] [--temperature 0] [--top-k 40] [--top-p 0.9] [--penalty 1.3]
 //          [--seed 0] [--ctx 2048] [--device 0]
-//   tl_run model.gguf --prompt "text" [--system "text"] [--qa 1] [...]      (needs the file's tokenizer metadata)
+//   tl_run MODEL --prompt "text" [--system "text"] [--qa 1] [...]      (needs the file's tokenizer metadata)
+// MODEL: a .gguf file (Llama family) or a checkpoint folder with config.json + model.safetensors (layer-list families,
+// token ids only); the family is chosen by the architecture the checkpoint names (tl_registry.hpp).
 // Prints one JSON line: {"generated": [...], "load_s": ..., "gen_s": ..., "tokens_per_s": ...}; with --prompt the
 // generated text follows on the next lines (the prompt goes through format_prompt / encode as in api.cpp:505-575).
 #include <chrono>
@@ -17,7 +19,7 @@
 
 int main(int argc, char** argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: %s model.gguf (--ids a,b,c | --prompt TEXT [--system TEXT] [--qa 1]) [--steps N] [--temperature T] [--top-k K] [--top-p P] "
+    fprintf(stderr, "usage: %s MODEL(.gguf file | checkpoint folder) (--ids a,b,c | --prompt TEXT [--system TEXT] [--qa 1]) [--steps N] [--temperature T] [--top-k K] [--top-p P] "
                     "[--penalty R] [--seed S] [--ctx C] [--device D]\n", argv[0]);
     return 2;
   }

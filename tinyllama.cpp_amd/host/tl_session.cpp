@@ -1,6 +1,8 @@
 // tl_session.cpp — see tl_session.hpp.
 #include "tl_session.hpp"
 
+#include "tl_registry.hpp"
+
 #include <algorithm>
 #include <chrono>
 #include <cmath>
@@ -87,19 +89,21 @@ ModelConfig config_from_gguf(const GGUFFile& f) {
   return c;
 }
 
-Session::Session(const std::string& model_path, int device, int max_context, int max_batch_size) {
+// The Llama family: one GGUF file (the reference's only checkpoint form for this backend).
+void load_llama_gguf(const std::string& model_path, int device, int max_context, LoadedModel* out) {
   const auto t0 = std::chrono::steady_clock::now();
   GGUFFile file;
   file.open(model_path);
+  ModelConfig& config_ = out->config;
+  LoadStats& stats_ = out->stats;
+  tl_model*& model_ = out->model;
   config_ = config_from_gguf(file);
   if (config_.hidden_size <= 0 || config_.num_hidden_layers <= 0 || config_.num_attention_heads <= 0 ||
       config_.intermediate_size <= 0)
     throw std::runtime_error("Session: " + model_path + " lacks the llama.* shape metadata");
   if (max_context > 0 && max_context < config_.max_position_embeddings) config_.max_position_embeddings = max_context;
-  if (max_batch_size < 1) throw std::runtime_error("Session: max_batch_size must be >= 1");
-  max_batch_size_ = max_batch_size;
   if (const GGUFValue* toks = file.meta("tokenizer.ggml.tokens"))
-    if (!toks->strings.empty()) tokenizer_.reset(new Tokenizer(file));
+    if (!toks->strings.empty()) out->tokenizer.reset(new Tokenizer(file));
   tl_check(tl_init(device), "tl_init");
   tl_model_config mc = {};
   mc.hidden_size = config_.hidden_size;
@@ -135,11 +139,75 @@ Session::Session(const std::string& model_path, int device, int max_context, int
     model_ = nullptr;
     throw;
   }
+  out->multi_sequence = true;
+  out->exact_terms = 6;
+  out->serving_terms = 0;
   stats_.seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
+
+Session::Session(const std::string& model_path, int device, int max_context, int max_batch_size) {
+  if (max_batch_size < 1) throw std::runtime_error("Session: max_batch_size must be >= 1");
+  max_batch_size_ = max_batch_size;
+  std::string container, resolved;
+  const std::string arch = detect_architecture(model_path, &container, &resolved);
+  const ModelFamily* family = find_model_family(arch, container);
+  if (!family) {
+    std::string known;
+    for (const ModelFamily& f : model_families()) known += std::string(known.empty() ? "" : ", ") + f.name;
+    throw std::runtime_error("Session: " + model_path + " names architecture \"" + arch + "\"; this build has " + known);
+  }
+  LoadedModel loaded;
+  family->load(resolved, device, max_context, &loaded);
+  config_ = loaded.config;
+  model_ = loaded.model;
+  tokenizer_ = std::move(loaded.tokenizer);
+  stats_ = loaded.stats;
+  multi_sequence_ = loaded.multi_sequence;
+  exact_terms_ = loaded.exact_terms;
+  serving_terms_ = loaded.serving_terms;
 }
 
 Session::~Session() {
   if (model_) tl_model_free(model_);
+}
+
+void Session::reset() { tl_check(tl_model_reset_kv(model_), "tl_model_reset_kv"); }
+
+void Session::set_exact(bool on) {
+  // min_batch 2: with an exact setting a caller compares portions of any length, so nothing but single tokens decodes
+  tl_check(tl_model_set_prefill(model_, on ? exact_terms_ : serving_terms_, on ? 2 : (multi_sequence_ ? 8 : 2)),
+           "tl_model_set_prefill");
+}
+
+std::vector<float> Session::forward(const std::vector<int>& tokens, int start_pos, const std::vector<int>& want) {
+  const int T = (int)tokens.size(), V = config_.vocab_size;
+  if (T == 0) throw std::runtime_error("Session::forward: no tokens");
+  if (start_pos < 0 || start_pos + T > config_.max_position_embeddings)
+    throw std::runtime_error("Session::forward: positions " + std::to_string(start_pos) + ".." + std::to_string(start_pos + T) +
+                             " exceed the cache of " + std::to_string(config_.max_position_embeddings));
+  for (size_t i = 0; i < want.size(); ++i)
+    if (want[i] < 0 || want[i] >= T || (i > 0 && want[i] <= want[i - 1]))
+      throw std::runtime_error("Session::forward: wanted rows must ascend inside the step");
+  std::vector<float> out(want.size() * (size_t)V);
+  if (T == 1 && start_pos > 0) {  // the decode step
+    tl_check(tl_model_decode(model_, tokens[0], start_pos, want.empty() ? nullptr : out.data(), nullptr), "tl_model_decode");
+    return out;
+  }
+  if (!multi_sequence_) {  // layer-list families return the chosen rows themselves
+    tl_check(tl_model_prefill_rows(model_, tokens.data(), T, start_pos, want.empty() ? nullptr : want.data(), (int)want.size(),
+                                   want.empty() ? nullptr : out.data()),
+             "tl_model_prefill_rows");
+    return out;
+  }
+  if (want.empty() || (want.size() == 1 && want[0] == T - 1)) {
+    tl_check(tl_model_prefill(model_, tokens.data(), T, start_pos, want.empty() ? nullptr : out.data(), nullptr), "tl_model_prefill");
+    return out;
+  }
+  std::vector<float> all((size_t)T * V);
+  tl_check(tl_model_prefill(model_, tokens.data(), T, start_pos, nullptr, all.data()), "tl_model_prefill");
+  for (size_t i = 0; i < want.size(); ++i)
+    std::copy(all.begin() + (size_t)want[i] * V, all.begin() + (size_t)(want[i] + 1) * V, out.begin() + i * (size_t)V);
+  return out;
 }
 
 std::vector<int> Session::generate(const std::vector<int>& prompt, int steps, float temperature, int top_k, float top_p) {
@@ -243,6 +311,23 @@ std::vector<std::vector<int>> Session::generate_batch(const std::vector<std::vec
   const int B = (int)prompts.size(), max_pos = config_.max_position_embeddings, V = config_.vocab_size;
   std::vector<std::vector<int>> out((size_t)B);
   if (steps <= 0) return out;
+  if (!multi_sequence_) {
+    // a family without the multi-sequence step: prompt by prompt, as the reference falls back to (api.cpp:1116-1130);
+    // no repetition penalty on this path either (api.cpp:993,1084)
+    const float keep = repetition_penalty_;
+    repetition_penalty_ = 1.0f;
+    try {
+      for (int i = 0; i < B; ++i) {
+        if (prompts[i].empty()) throw std::runtime_error("Session::generate_batch: empty prompt");
+        out[i] = generate(prompts[i], steps, temperature, top_k, top_p);
+      }
+    } catch (...) {
+      repetition_penalty_ = keep;
+      throw;
+    }
+    repetition_penalty_ = keep;
+    return out;
+  }
   for (const auto& p : prompts) {
     if (p.empty()) throw std::runtime_error("Session::generate_batch: empty prompt (the reference substitutes BOS after tokenizing, api.cpp:912-915)");
     if ((int)p.size() > max_pos) throw std::runtime_error("Session::generate_batch: prompt longer than the context");

@@ -35,7 +35,8 @@ struct LoadStats {
 
 class Session {
  public:
-  // model_path: a .gguf file. device: HIP device ordinal. max_context > 0 caps the KV cache length below the file's
+  // model_path: a .gguf file, or a checkpoint folder (config.json + model.safetensors; the config.json itself also does):
+  // the model family is chosen by the architecture the checkpoint names (tl_registry.hpp). device: HIP device ordinal. max_context > 0 caps the KV cache length below the file's
   // context length. tp_rank / tp_size: tensor-parallel shard (the caller wires the communicator through model()).
   // max_batch_size: most prompts one generate_batch() call may carry (api.h:39-46; 1 = single-sequence use only).
   explicit Session(const std::string& model_path, int device = 0, int max_context = 0, int max_batch_size = 1);
@@ -68,6 +69,15 @@ class Session {
   // null when the file has no tokenizer.ggml.tokens (the synthetic test models)
   const Tokenizer* get_tokenizer() const { return tokenizer_.get(); }
 
+  // The step function on token ids, for callers that schedule themselves (tl_trace replays recorded steps through it):
+  // feeds `tokens` at positions start_pos.. on top of what earlier calls left in the cache and returns the logits of the
+  // token rows listed in `want` (ascending), [want.size()][vocab]. One token at a position > 0 is the decode step (the
+  // captured graph); anything else goes through the batched prefill. reset() gives the cache back for the next sequence.
+  std::vector<float> forward(const std::vector<int>& tokens, int start_pos, const std::vector<int>& want);
+  void reset();
+  // true: the prompt-chunk GEMMs run FP32-grade (every family has such a setting); false: the family's serving default
+  void set_exact(bool on);
+
   void set_max_batch_size(int n);
   int get_max_batch_size() const { return max_batch_size_; }
   void set_repetition_penalty(float p) { repetition_penalty_ = p; }
@@ -85,6 +95,8 @@ class Session {
   float repetition_penalty_ = 1.3f;  // api.h:135
   int max_batch_size_ = 1;           // api.h:142
   int batch_ready_ = 0;              // sequences the device-side batch cache was sized for
+  bool multi_sequence_ = true;       // the family has the multi-sequence decode step (else generate_batch goes prompt by prompt)
+  int exact_terms_ = 6, serving_terms_ = 0;
   LoadStats stats_;
 };
 

@@ -33,6 +33,10 @@ SIGNATURES = {
     "tlh_session_set_max_batch": [_vp, _i],
     "tlh_session_generate_batch": [_vp, _vp, _vp, _i, _i, _f, _i, _f, _vp, _vp],
     "tlh_session_load_stats": [_vp, _vp, _vp, _vp],
+    "tlh_session_forward": [_vp, _vp, _i, _i, _vp, _i, _vp],
+    "tlh_session_reset": [_vp],
+    "tlh_session_set_exact": [_vp, _i],
+    "tlh_session_info": [_vp, _vp, C.c_char_p, C.c_size_t],
     "tlh_tokenizer_from_gguf": [_vp, _i, _vp],
     "tlh_tokenizer_close": [_vp],
     "tlh_tokenizer_info": [_vp, _vp],
@@ -250,6 +254,30 @@ class Session:
                                                len(prompts), int(steps), float(temperature), int(top_k), float(top_p),
                                                out.ctypes.data, lens.ctypes.data), "tlh_session_generate_batch")
         return [out[i, : lens[i]].copy() for i in range(len(prompts))]
+
+    def info(self):
+        """{"vocab", "width", "layers", "max_pos", "architecture"} of the opened model."""
+        out = (C.c_int * 4)()
+        buf = C.create_string_buffer(128)
+        check(lib().tlh_session_info(self.h, out, buf, 128), "tlh_session_info")
+        return {"vocab": out[0], "width": out[1], "layers": out[2], "max_pos": out[3], "architecture": buf.value.decode()}
+
+    def forward(self, tokens, start_pos=0, want=None):
+        """Session::forward: logits [len(want), vocab] of the token rows `want` (None: all) of this step."""
+        toks = np.ascontiguousarray(tokens, np.int32)
+        want = np.arange(toks.size, dtype=np.int32) if want is None else np.ascontiguousarray(want, np.int32)
+        if not hasattr(self, "_vocab"):
+            self._vocab = self.info()["vocab"]
+        out = np.empty((want.size, self._vocab), np.float32)
+        check(lib().tlh_session_forward(self.h, toks.ctypes.data, toks.size, int(start_pos), want.ctypes.data, want.size,
+                                        out.ctypes.data), "tlh_session_forward")
+        return out
+
+    def reset(self):
+        check(lib().tlh_session_reset(self.h), "tlh_session_reset")
+
+    def set_exact(self, on=True):
+        check(lib().tlh_session_set_exact(self.h, int(bool(on))), "tlh_session_set_exact")
 
     def load_stats(self):
         a, b, c = C.c_uint64(), C.c_uint64(), C.c_double()
