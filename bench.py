@@ -52,6 +52,11 @@ def parse():
     ap.add_argument("--prompt-len", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers in the CPU-baseline sample")
+    ap.add_argument("--family", default=None, choices=[None, "ralasun"],
+                    help="ralasun: prefill / decode throughput of the layer-list family at --sizes beside a Llama model of "
+                         "equal size (one GPU; prints its own JSON line; the default workload and line are untouched)")
+    ap.add_argument("--sizes", default="s,m,l", help="with --family: comma-separated names out of s, m, l")
+    ap.add_argument("--prefill-tokens", type=int, default=2048, help="with --family: prompt length of the prefill leg")
     return ap.parse_args()
 
 
@@ -88,8 +93,141 @@ def dist_setup(n_gpus):
     return rank, world, local, dist
 
 
+# ---- layer-list family beside the closest Llama model (--family ralasun) ---------------------------------------------------
+# Sizes that resemble real layers. The Llama twin has the same width, heads, layers, vocabulary and as many feed-forward
+# columns as one token activates here (top * expert ff + shared ff), stored Q8_0 (the closest of its formats to bf16).
+STACK_SIZES = {
+    "s": dict(width=1024, layers=8, heads=16, kv_heads=4, dim=64, vdim=64, window=512, experts=8, top=2, ff=512,
+              shared_ff=1024, vocab=32000),
+    "m": dict(width=2048, layers=12, heads=32, kv_heads=8, dim=64, vdim=64, window=1024, experts=16, top=4, ff=768,
+              shared_ff=1024, vocab=32000),
+    "l": dict(width=4096, layers=6, heads=32, kv_heads=8, dim=128, vdim=128, window=2048, experts=16, top=4, ff=1024,
+              shared_ff=2048, vocab=64000),
+}
+
+
+def _pool_bf16(S, n, std, rng, pool):
+    """n bf16 values of roughly N(0, std^2) cut out of a shared random pool (building billions of normals takes minutes)."""
+    off = int(rng.integers(0, pool.size))
+    reps = -(-(n + off) // pool.size)
+    a = np.tile(pool, reps)[off:off + n] if reps > 1 else pool[off:off + n]
+    return S.to_bf16(a * np.float32(std))
+
+
+def stack_bench(args):
+    from _pkg import load_package
+    pkg = load_package()
+    S = pkg.synth
+    from tinyllama_cpp_amd import engine
+    engine.init(0)
+    rng = np.random.default_rng(0)
+    pool = rng.standard_normal(1 << 22).astype(np.float32)
+    T = args.prefill_tokens
+    results = []
+    for name in [x for x in args.sizes.split(",") if x]:
+        z = STACK_SIZES[name]
+        W, V = z["width"], z["vocab"]
+        layer = S.stack_layer(z["heads"], z["kv_heads"], z["dim"], z["vdim"], z["window"], v_mix=True, experts=z["experts"],
+                              top=z["top"], ff=z["ff"], shared_ff=z["shared_ff"])
+        cfg = S.stack_config(W, V, [layer] * z["layers"])
+        max_pos = T + args.steps + args.warmup + 64
+        m = engine.StackModel(cfg, max_pos)
+
+        def mat(nm, r, c, std=None):
+            m.set_tensor(nm, _pool_bf16(S, r * c, std or 1.0 / np.sqrt(c), rng, pool).reshape(r, c))
+
+        def vec(nm, n, centre):
+            m.set_tensor(nm, S.to_bf16((centre + 0.05 * rng.standard_normal(n)).astype(np.float32)))
+
+        t0 = time.time()
+        mat("embed", V, W, 1.0), mat("head", V, W), vec("embed.norm", W, 0.0), vec("final.norm", W, 0.0)
+        for i in range(z["layers"]):
+            p = f"l{i}."
+            qd, kd, vd, od = z["heads"] * z["dim"], z["kv_heads"] * z["dim"], z["kv_heads"] * z["vdim"], z["heads"] * z["vdim"]
+            mat(p + "mix.q", qd, W), mat(p + "mix.k", kd, W), mat(p + "mix.v", vd, W), mat(p + "mix.o", W, od)
+            vec(p + "mix.q.norm", qd, 1.0), vec(p + "mix.k.norm", kd, 1.0), vec(p + "norm1", W, 0.0), vec(p + "norm2", W, 0.0)
+            m.set_tensor(p + "mix.vmix", S.to_bf16(np.array(0.5, np.float32)))
+            mat(p + "mlp.router", z["experts"], W), vec(p + "mlp.router.b", z["experts"], 0.0)
+            for e in range(z["experts"]):
+                mat(p + f"mlp.e{e}.gate", z["ff"], W), mat(p + f"mlp.e{e}.up", z["ff"], W), mat(p + f"mlp.e{e}.down", W, z["ff"])
+            mat(p + "mlp.shared.gate", z["shared_ff"], W), mat(p + "mlp.shared.up", z["shared_ff"], W)
+            mat(p + "mlp.shared.down", W, z["shared_ff"])
+        m.finalize()
+        load_s = time.time() - t0
+        toks = rng.integers(0, V, T).astype(np.int32)
+        last_row = np.array([T - 1], np.int32)
+        r = {"size": name, "shape": z, "load_s": round(load_s, 1)}
+        per_tok = (z["heads"] * z["dim"] + z["kv_heads"] * (z["dim"] + z["vdim"]) + z["heads"] * z["vdim"]) * W \
+            + 3 * W * (z["top"] * z["ff"] + z["shared_ff"]) + W * z["experts"]
+        for terms, label in ((1, "bf16"), (3, "fp32_grade")):
+            m.set_prefill(terms, 1)
+            m.reset_kv()
+            m.prefill_rows(toks, 0, last_row)
+            best = 1e9
+            for _ in range(3):
+                m.reset_kv()
+                t0 = time.perf_counter()
+                m.prefill_rows(toks, 0, last_row)
+                best = min(best, time.perf_counter() - t0)
+            r[f"prefill_{label}_tokens_per_s"] = round(T / best, 1)
+            r[f"prefill_{label}_gemm_tflops"] = round(2.0 * T * per_tok * z["layers"] / best / 1e12, 2)
+        m.set_prefill(1, 1)
+        first = int(np.argmax(m.prefill_rows(toks, 0, last_row)[0]))  # the cache now holds T positions
+        m.generate_greedy(first, T, args.warmup)
+        t0 = time.perf_counter()
+        m.generate_greedy(first, T + args.warmup, args.steps)
+        dt = time.perf_counter() - t0
+        wb, kb = m.bytes_per_token(T + args.warmup)
+        r.update(decode_tokens_per_s=round(args.steps / dt, 1), decode_us_per_token=round(dt / args.steps * 1e6, 1),
+                 decode_bytes_per_token=int(wb + kb), decode_hbm_gbps=round((wb + kb) * args.steps / dt / 1e9, 1),
+                 decode_frac_of_hbm_peak=round((wb + kb) * args.steps / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                 graph_nodes=m.graph_nodes())
+        m.free()
+        # ---- the Llama twin ------------------------------------------------------------------------------------------
+        lc = dict(hidden=W, inter=z["top"] * z["ff"] + z["shared_ff"], n_heads=z["heads"], n_kv_heads=z["kv_heads"],
+                  n_layers=z["layers"], vocab=V, max_pos=max_pos, eps=1e-5, rope_theta=10000.0)
+        if W // z["heads"] == z["dim"] and z["dim"] == z["vdim"]:
+            lm = engine.Model(lc)
+            for nm, typ, rows, cols in S.tensor_plan(lc, "q8_0"):
+                lm.set_tensor(nm, typ, S.make_tensor(nm, typ, rows, cols, 42), rows, cols)
+            lm.finalize()
+            tw = {"format": "q8_0", "shape": {k: lc[k] for k in ("hidden", "inter", "n_heads", "n_kv_heads", "n_layers", "vocab")}}
+            lper = sum(rr * cc for n_, t_, rr, cc in S.tensor_plan(lc, "q8_0") if n_.startswith("blk.0.") and t_ != S.F32)
+            for terms, label in ((1, "bf16"), (6, "fp32_grade")):
+                lm.set_prefill(terms=terms, min_batch=8)
+                lm.reset_kv()
+                lm.prefill(toks, 0)
+                best = 1e9
+                for _ in range(3):
+                    lm.reset_kv()
+                    t0 = time.perf_counter()
+                    lm.prefill(toks, 0)
+                    best = min(best, time.perf_counter() - t0)
+                tw[f"prefill_{label}_tokens_per_s"] = round(T / best, 1)
+                tw[f"prefill_{label}_gemm_tflops"] = round(2.0 * T * lper * z["layers"] / best / 1e12, 2)
+            lm.generate_greedy(first, T, args.warmup)
+            t0 = time.perf_counter()
+            lm.generate_greedy(first, T + args.warmup, args.steps)
+            dt = time.perf_counter() - t0
+            wb, kb = lm.bytes_per_token(T + args.warmup)
+            tw.update(decode_tokens_per_s=round(args.steps / dt, 1), decode_us_per_token=round(dt / args.steps * 1e6, 1),
+                      decode_bytes_per_token=int(wb + kb), decode_hbm_gbps=round((wb + kb) * args.steps / dt / 1e9, 1),
+                      decode_frac_of_hbm_peak=round((wb + kb) * args.steps / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                      graph_nodes=lm.graph_nodes())
+            lm.free()
+            r["llama_twin"] = tw
+        results.append(r)
+        print(json.dumps(r), file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "layer-list family (Ralasun): prefill / decode tokens/s beside a Llama model of equal size",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "prefill_tokens": T, "dtype": "bf16 weights, "
+                      "fp32 activations", "data": "synthetic", "results": results}))
+    return 0
+
+
 def main():
     args = parse()
+    if args.family:
+        return stack_bench(args)
     # Watchdog (seconds; TL_BENCH_WATCHDOG, 900 by default for multi-rank runs): dump every thread's Python stack to stderr
     # and exit instead of sitting in a collective for ever. Multi-rank runs also shorten the peer exchange's poll deadline
     # (5 s by default in the library): the ranks enter every collective call together here (barriers in front of finalize),

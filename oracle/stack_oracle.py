@@ -103,7 +103,7 @@ class StackOracle:
                 if v_first is None:
                     v_first = v
                 else:
-                    lam = float(w[p + "vmix"])
+                    lam = float(np.asarray(w[p + "vmix"]).reshape(-1)[0])
                     v = (1.0 - lam) * v + lam * v_first
             self.k[i] = k if self.k[i] is None else np.concatenate([self.k[i], k])
             self.v[i] = v if self.v[i] is None else np.concatenate([self.v[i], v])

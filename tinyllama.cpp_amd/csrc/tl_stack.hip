@@ -369,6 +369,11 @@ void tl_stack_bytes_per_token(const TlStack* st, int pos, double* weight_bytes, 
 
 namespace {
 
+// One token is always FP32-grade: the decode step's GEMVs are, and where TL_STACK_GEMV=0 sends it through the chunk GEMMs
+// instead (a test configuration) it takes three terms, whatever the chunks use; so the captured step never depends on a
+// setting that may change after the capture.
+inline int terms_for(const TlStack* st, int T) { return T == 1 ? 3 : st->terms; }
+
 // y[T][rows] = x[T][cols] W^T for a chunk, or the GEMV for the one token of a decode step
 int project(TlStack* st, const uint16_t* w, int rows, int cols, const float* x, int ldx, float* y, int ldy, int T,
             hipStream_t s) {
@@ -382,7 +387,7 @@ int project(TlStack* st, const uint16_t* w, int rows, int cols, const float* x, 
   d.y = y;
   d.ldy = ldy;
   d.T = T;
-  d.terms = st->terms;
+  d.terms = terms_for(st, T);
   return tl_launch_dense_gemm(d, s);
 }
 
@@ -438,7 +443,7 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
   g.y = st->gu_buf;
   g.ldy = 2 * ff;
   g.T = S;
-  g.terms = st->terms;
+  g.terms = terms_for(st, T);
   g.x_rows = st->slot_of;
   g.x_div = sp.top;
   g.groups = sp.experts;
@@ -454,7 +459,7 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
   d.y = st->eout;
   d.ldy = W;
   d.T = S;
-  d.terms = st->terms;
+  d.terms = terms_for(st, T);
   d.y_rows = st->slot_of;
   d.groups = sp.experts;
   d.group_off = st->off;
