@@ -11,6 +11,7 @@
 //   A workgroup of 4 waves owns a 64-feature x 64-token tile, BK = 32. Items may be gathered (x_rows), scattered (y_rows) and
 //   grouped (group_off: blockIdx.z = matrix of the group; tiles beyond a group's items leave at once), which is what the
 //   experts of a mixture need: the plan lives on the device, the grid is sized for the worst case.
+#include "tl_bf16.h"
 #include "tl_stack.h"
 
 namespace {
@@ -23,7 +24,7 @@ __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest e
   u += 0x7fffu + ((u >> 16) & 1u);
   return (unsigned short)(u >> 16);
 }
-__device__ __forceinline__ float bf2f(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+__device__ __forceinline__ float bf2f(unsigned short h) { return tl_bf2f(h); }
 
 constexpr int BM = 64, BN = 64, BK = 32, LDK = 40;  // LDK: padded row of a tile in LDS (80 B, keeps 16 B / 8 B alignment)
 
@@ -135,29 +136,20 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
   }
 }
 
+// RW rows per wave, 4 waves per workgroup: 2 x RW sixteen-byte weight loads in flight per lane (tl_bf16.h)
+template <int RW>
 __global__ __launch_bounds__(256) void dense_gemv_kernel(const unsigned short* __restrict__ W, int rows, int cols,
                                                          const float* __restrict__ x, float* __restrict__ y, int vec) {
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const unsigned short* wr = W + (size_t)row * cols;
-  float s = 0.0f;
-  if (vec) {
-    for (int k = lane * 8; k < cols; k += 512) {
-      const uint4 w4 = *reinterpret_cast<const uint4*>(wr + k);
-      const float4 x0 = *reinterpret_cast<const float4*>(x + k);
-      const float4 x1 = *reinterpret_cast<const float4*>(x + k + 4);
-      s += __uint_as_float(w4.x << 16) * x0.x + __uint_as_float(w4.x & 0xffff0000u) * x0.y +
-           __uint_as_float(w4.y << 16) * x0.z + __uint_as_float(w4.y & 0xffff0000u) * x0.w +
-           __uint_as_float(w4.z << 16) * x1.x + __uint_as_float(w4.z & 0xffff0000u) * x1.y +
-           __uint_as_float(w4.w << 16) * x1.z + __uint_as_float(w4.w & 0xffff0000u) * x1.w;
-    }
-  } else {
-    for (int k = lane; k < cols; k += 64) s += bf2f(wr[k]) * x[k];
-  }
+  const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
+  if (row0 >= rows) return;
+  float out[RW];
+  tl_wave_dot_rows<RW>(W + (size_t)row0 * cols, (size_t)cols, rows - row0, x, cols, vec != 0, lane, out);
+  if (lane == 0) {
 #pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
-  if (lane == 0) y[row] = s;
+    for (int r = 0; r < RW; ++r)
+      if (row0 + r < rows) y[row0 + r] = out[r];
+  }
 }
 
 }  // namespace
@@ -179,7 +171,11 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
 int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s) {
   TL_REQUIRE(w && x && y && rows > 0 && cols > 0, "dense gemv: bad arguments");
   const int vec = (cols & 7) == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0;
-  dense_gemv_kernel<<<(rows + 3) / 4, 256, 0, s>>>(w, rows, cols, x, y, vec);
+  // rows per wave: as many as still leave every CU a few workgroups
+  const int cus = tl_num_cus();
+  if (rows >= 16 * 4 * cus) dense_gemv_kernel<4><<<(rows + 15) / 16, 256, 0, s>>>(w, rows, cols, x, y, vec);
+  else if (rows >= 8 * 4 * cus) dense_gemv_kernel<2><<<(rows + 7) / 8, 256, 0, s>>>(w, rows, cols, x, y, vec);
+  else dense_gemv_kernel<1><<<(rows + 3) / 4, 256, 0, s>>>(w, rows, cols, x, y, vec);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -12,41 +12,28 @@
 //            router weights (and the shared expert's with weight 1).
 #include <math.h>
 
+#include "tl_bf16.h"
 #include "tl_stack.h"
 
 namespace {
 
 constexpr int kMaxExperts = 1024;
 
-__device__ __forceinline__ float bf2f(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
-
 // dot of a bf16 row with an FP32 vector over the lanes of a wave; result in every lane
 __device__ __forceinline__ float wave_dot(const unsigned short* __restrict__ wr, const float* __restrict__ x, int n, bool vec,
                                           int lane) {
-  float s = 0.0f;
-  if (vec) {
-    for (int k = lane * 8; k < n; k += 512) {
-      const uint4 w4 = *reinterpret_cast<const uint4*>(wr + k);
-      const float4 x0 = *reinterpret_cast<const float4*>(x + k);
-      const float4 x1 = *reinterpret_cast<const float4*>(x + k + 4);
-      s += __uint_as_float(w4.x << 16) * x0.x + __uint_as_float(w4.x & 0xffff0000u) * x0.y +
-           __uint_as_float(w4.y << 16) * x0.z + __uint_as_float(w4.y & 0xffff0000u) * x0.w +
-           __uint_as_float(w4.z << 16) * x1.x + __uint_as_float(w4.z & 0xffff0000u) * x1.y +
-           __uint_as_float(w4.w << 16) * x1.z + __uint_as_float(w4.w & 0xffff0000u) * x1.w;
-    }
-  } else {
-    for (int k = lane; k < n; k += 64) s += bf2f(wr[k]) * x[k];
-  }
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
+  float s;
+  tl_wave_dot_rows<1>(wr, 0, 1, x, n, vec, lane, &s);
   return s;
 }
 
-__global__ __launch_bounds__(256) void router_kernel(const RouterArgs a, int vec) {
+// 4 or 16 waves per token: a wave takes every (number of waves)-th expert
+__global__ __launch_bounds__(1024) void router_kernel(const RouterArgs a, int vec) {
   extern __shared__ float z[];  // [experts]
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float* x = a.x + (size_t)t * a.width;
-  for (int e = wave; e < a.experts; e += 4) {
+  const int nwaves = blockDim.x >> 6;
+  for (int e = wave; e < a.experts; e += nwaves) {
     const float s = wave_dot(a.w + (size_t)e * a.width, x, a.width, vec != 0, lane);
     if (lane == 0) z[e] = s + (a.b ? a.b[e] : 0.0f);
   }
@@ -143,9 +130,9 @@ __global__ __launch_bounds__(256) void moe_decode_gu_kernel(const MoeDecodeArgs 
   const int ff = shared ? a.sff : a.ff;
   if (r >= ff) return;
   const unsigned short* gu = shared ? a.sgu : a.gu + (size_t)a.ids[j] * 2 * a.ff * a.width;
-  const float g = wave_dot(gu + (size_t)r * a.width, a.x, a.width, vec != 0, lane);
-  const float u = wave_dot(gu + (size_t)(ff + r) * a.width, a.x, a.width, vec != 0, lane);
-  if (lane == 0) a.act[(size_t)j * a.ff + r] = glu_act(g, u, shared ? a.slimit : a.limit, a.alpha);
+  float gu2[2];  // row r of the gate and of the up matrix, their loads in flight together
+  tl_wave_dot_rows<2>(gu + (size_t)r * a.width, (size_t)ff * a.width, 2, a.x, a.width, vec != 0, lane, gu2);
+  if (lane == 0) a.act[(size_t)j * a.ff + r] = glu_act(gu2[0], gu2[1], shared ? a.slimit : a.limit, a.alpha);
 }
 
 __global__ __launch_bounds__(256) void moe_decode_down_kernel(const MoeDecodeArgs a, int vec_e, int vec_s) {
@@ -167,7 +154,8 @@ int tl_launch_router(const RouterArgs& a, hipStream_t s) {
   TL_REQUIRE(a.experts > 0 && a.experts <= kMaxExperts, "router: %d experts outside (0, %d]", a.experts, kMaxExperts);
   TL_REQUIRE(a.top > 0 && a.top <= a.experts, "router: top %d of %d experts", a.top, a.experts);
   const int vec = (a.width & 7) == 0 && ((size_t)a.x & 15) == 0 && ((size_t)a.w & 15) == 0;
-  router_kernel<<<a.T, 256, sizeof(float) * a.experts, s>>>(a, vec);
+  // few tokens (the decode step): the experts' rows are latency-bound round trips, so spread them over 16 waves
+  router_kernel<<<a.T, a.T <= 8 && a.experts > 4 ? 1024 : 256, sizeof(float) * a.experts, s>>>(a, vec);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -1,42 +1,49 @@
 // tl_norm.hip — the row-wise FP32 steps between the matrix products of a layer-list model. Every norm here is
 // y = x / sqrt(mean(x^2) + eps) * weight, eps inside the root; "one-plus" weights are stored around zero and applied as
-// (1 + w). One workgroup of 256 threads per token row; a row is staged in LDS, so that it is read from memory once.
+// (1 + w). One workgroup per token row (256 threads for the rows of a prompt chunk, 1024 for the few rows of a decode step,
+// whose launches are nothing but a chain of memory round trips); a row is staged in LDS, so that it is read from memory once.
 #include <math.h>
 
 #include "tl_stack.h"
 
 namespace {
 
-__device__ __forceinline__ float block_sum(float v, float* red) {  // red: >= 4 floats of LDS; result in every thread
+constexpr int kMaxWaves = 16;
+
+__device__ __forceinline__ float block_sum(float v, float* red) {  // red: kMaxWaves floats of LDS; result in every thread
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
+  float s = 0.0f;
+  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) s += red[w];  // in wave order: the same sum in every thread
+  return s;
 }
 
-__global__ __launch_bounds__(256) void embed_norm_kernel(const unsigned short* __restrict__ table, int vocab, int width,
+inline int row_threads(int rows) { return rows <= 8 ? 1024 : 256; }
+
+__global__ __launch_bounds__(1024) void embed_norm_kernel(const unsigned short* __restrict__ table, int vocab, int width,
                                                          const int* __restrict__ tokens, const float* __restrict__ w,
                                                          float eps, float* __restrict__ x) {
   extern __shared__ float row[];
-  __shared__ float red[4];
+  __shared__ float red[kMaxWaves];
   const int t = blockIdx.x, tok = tokens[t];
   const bool in = tok >= 0 && tok < vocab;
   const unsigned short* e = table + (size_t)(in ? tok : 0) * width;
   float ss = 0.0f;
-  for (int c = threadIdx.x; c < width; c += 256) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float v = in ? __uint_as_float((unsigned)e[c] << 16) : 0.0f;
     row[c] = v;
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int c = threadIdx.x; c < width; c += 256) x[(size_t)t * width + c] = row[c] * inv * (1.0f + w[c]);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) x[(size_t)t * width + c] = row[c] * inv * (1.0f + w[c]);
 }
 
-__global__ __launch_bounds__(256) void qkv_post_kernel(const QkvPostArgs a) {
-  __shared__ float red[4];
+__global__ __launch_bounds__(1024) void qkv_post_kernel(const QkvPostArgs a) {
+  __shared__ float red[kMaxWaves];
   const int t = blockIdx.x;
   const int pos = (a.pos_dev ? *a.pos_dev : a.start_pos) + t;
   float* q = a.qkv + (size_t)t * a.ld;
@@ -44,40 +51,40 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(const QkvPostArgs a) {
   const float* v = k + a.kd;
   float sq = 0.0f, sk = 0.0f;
   if (a.q_norm)
-    for (int c = threadIdx.x; c < a.qd; c += 256) sq += q[c] * q[c];
+    for (int c = threadIdx.x; c < a.qd; c += blockDim.x) sq += q[c] * q[c];
   if (a.k_norm)
-    for (int c = threadIdx.x; c < a.kd; c += 256) sk += k[c] * k[c];
+    for (int c = threadIdx.x; c < a.kd; c += blockDim.x) sk += k[c] * k[c];
   sq = block_sum(sq, red);
   sk = block_sum(sk, red);
   if (a.q_norm) {
     const float inv = 1.0f / sqrtf(sq / (float)a.qd + a.eps);
-    for (int c = threadIdx.x; c < a.qd; c += 256) q[c] = q[c] * inv * a.q_norm[c];
+    for (int c = threadIdx.x; c < a.qd; c += blockDim.x) q[c] = q[c] * inv * a.q_norm[c];
   }
   {
     const float inv = a.k_norm ? 1.0f / sqrtf(sk / (float)a.kd + a.eps) : 1.0f;
     float* kr = a.kc + (size_t)pos * a.kd;
-    for (int c = threadIdx.x; c < a.kd; c += 256) kr[c] = a.k_norm ? k[c] * inv * a.k_norm[c] : k[c];
+    for (int c = threadIdx.x; c < a.kd; c += blockDim.x) kr[c] = a.k_norm ? k[c] * inv * a.k_norm[c] : k[c];
   }
   float* vr = a.vc + (size_t)pos * a.vd;
   if (a.vmix == 2) {
     const float lam = *a.lambda;
     const float* vf = a.v_first + (size_t)t * a.vd;
-    for (int c = threadIdx.x; c < a.vd; c += 256) vr[c] = (1.0f - lam) * v[c] + lam * vf[c];
+    for (int c = threadIdx.x; c < a.vd; c += blockDim.x) vr[c] = (1.0f - lam) * v[c] + lam * vf[c];
   } else {
     float* vf = a.vmix == 1 ? a.v_first + (size_t)t * a.vd : nullptr;
-    for (int c = threadIdx.x; c < a.vd; c += 256) {
+    for (int c = threadIdx.x; c < a.vd; c += blockDim.x) {
       vr[c] = v[c];
       if (vf) vf[c] = v[c];
     }
   }
 }
 
-__global__ __launch_bounds__(256) void resid_norm_kernel(const ResidNormArgs a) {
+__global__ __launch_bounds__(1024) void resid_norm_kernel(const ResidNormArgs a) {
   extern __shared__ float row[];
-  __shared__ float red[4];
+  __shared__ float red[kMaxWaves];
   const int t = blockIdx.x;
   float ss = 0.0f;
-  for (int c = threadIdx.x; c < a.width; c += 256) {
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
     float y = a.a ? a.a[(size_t)t * a.width + c] : 0.0f;
     if (a.slots) {
       float e = 0.0f;
@@ -90,24 +97,24 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(const ResidNormArgs a) 
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)a.width + a.eps);
   float* x = a.x + (size_t)t * a.width;
-  for (int c = threadIdx.x; c < a.width; c += 256) x[c] += row[c] * inv * (1.0f + a.w[c]);
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) x[c] += row[c] * inv * (1.0f + a.w[c]);
 }
 
-__global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict__ x, int width, const int* __restrict__ rows,
+__global__ __launch_bounds__(1024) void norm_rows_kernel(const float* __restrict__ x, int width, const int* __restrict__ rows,
                                                         const float* __restrict__ w, float eps, float* __restrict__ out) {
   extern __shared__ float row[];
-  __shared__ float red[4];
+  __shared__ float red[kMaxWaves];
   const int i = blockIdx.x;
   const float* xr = x + (size_t)(rows ? rows[i] : i) * width;
   float ss = 0.0f;
-  for (int c = threadIdx.x; c < width; c += 256) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
     const float v = xr[c];
     row[c] = v;
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int c = threadIdx.x; c < width; c += 256) out[(size_t)i * width + c] = row[c] * inv * (1.0f + w[c]);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)i * width + c] = row[c] * inv * (1.0f + w[c]);
 }
 
 constexpr int kMaxRowFloats = 16 * 1024;  // 64 KB of LDS for the staged row
@@ -118,7 +125,7 @@ int tl_launch_embed_norm(const uint16_t* table, int vocab, int width, const int*
                          float* x, hipStream_t s) {
   TL_REQUIRE(table && tokens_dev && w && x && T > 0 && vocab > 0, "embed_norm: bad arguments");
   TL_REQUIRE(width > 0 && width <= kMaxRowFloats, "embed_norm: width %d outside (0, %d]", width, kMaxRowFloats);
-  embed_norm_kernel<<<T, 256, sizeof(float) * width, s>>>(table, vocab, width, tokens_dev, w, eps, x);
+  embed_norm_kernel<<<T, row_threads(T), sizeof(float) * width, s>>>(table, vocab, width, tokens_dev, w, eps, x);
   TL_HIP(hipGetLastError());
   return 0;
 }
@@ -128,7 +135,7 @@ int tl_launch_qkv_post(const QkvPostArgs& a, hipStream_t s) {
              "qkv_post: bad arguments");
   TL_REQUIRE(a.vmix == 0 || a.v_first, "qkv_post: value mixing without a v_first buffer");
   TL_REQUIRE(a.vmix != 2 || a.lambda, "qkv_post: value mixing without its coefficient");
-  qkv_post_kernel<<<a.T, 256, 0, s>>>(a);
+  qkv_post_kernel<<<a.T, row_threads(a.T), 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }
@@ -137,7 +144,7 @@ int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s) {
   TL_REQUIRE(a.x && a.w && a.T > 0 && (a.a || a.slots), "resid_norm: bad arguments");
   TL_REQUIRE(a.width > 0 && a.width <= kMaxRowFloats, "resid_norm: width %d outside (0, %d]", a.width, kMaxRowFloats);
   TL_REQUIRE(!a.slots || (a.slot_w && a.top > 0), "resid_norm: expert slots without weights");
-  resid_norm_kernel<<<a.T, 256, sizeof(float) * a.width, s>>>(a);
+  resid_norm_kernel<<<a.T, row_threads(a.T), sizeof(float) * a.width, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }
@@ -146,7 +153,7 @@ int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, c
                         hipStream_t s) {
   TL_REQUIRE(x && w && out && n > 0, "norm_rows: bad arguments");
   TL_REQUIRE(width > 0 && width <= kMaxRowFloats, "norm_rows: width %d outside (0, %d]", width, kMaxRowFloats);
-  norm_rows_kernel<<<n, 256, sizeof(float) * width, s>>>(x, width, rows_dev, w, eps, out);
+  norm_rows_kernel<<<n, row_threads(n), sizeof(float) * width, s>>>(x, width, rows_dev, w, eps, out);
   TL_HIP(hipGetLastError());
   return 0;
 }

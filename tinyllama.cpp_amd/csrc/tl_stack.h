@@ -44,8 +44,14 @@ struct SwaArgs {
   float scale;
   int start_pos;    // position of token 0 ...
   const int* pos_dev;  // ... or, when set, read from the device (graph replay)
+  // nsplit > 1: the visible keys of a (token, head) are dealt to nsplit workgroups whose partial results meet in ws
+  // (tl_swa_ws_floats floats) and are combined by a second small launch: the decode step's way to fill the chip
+  int nsplit;
+  float* ws;
 };
 int tl_launch_swa(const SwaArgs& a, hipStream_t s);
+int tl_swa_splits(int T, int window, int max_pos);  // splits worth having for T tokens over a cache of max_pos rows
+size_t tl_swa_ws_floats(int T, int heads, int vdim, int nsplit);
 
 // ---- tl_norm.hip -------------------------------------------------------------------------------------------------------
 // x[t] = embed[token[t]] / rms * (1 + w)   (bf16 table; an id outside the table embeds as zeros)

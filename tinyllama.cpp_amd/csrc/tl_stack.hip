@@ -54,6 +54,7 @@ struct TlStack {
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
   float *gu_buf = nullptr, *act_buf = nullptr, *eout = nullptr, *sgu_buf = nullptr, *sact = nullptr, *sout = nullptr;
   float* wts = nullptr;
+  float* swa_ws = nullptr;  // partial results of split attention launches (few tokens, long windows)
   int *ids = nullptr, *off = nullptr, *slot_of = nullptr;
   int max_qkv = 0, max_od = 0, max_vd = 0, max_top = 0, max_experts = 0, max_gu = 0, max_sff = 0;
   tl_stack_layer_hook hook = nullptr;
@@ -304,6 +305,15 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
   TL_TRY(dev_alloc(st, &st->proj, C * W));
   TL_TRY(dev_alloc(st, &st->v_first, C * st->max_vd));
   TL_TRY(dev_alloc(st, &st->xn, C * W));
+  {
+    size_t ws = 1;
+    for (const Layer& L : st->layers)
+      for (int T = 1; T <= 4; ++T) {
+        const size_t n = tl_swa_ws_floats(T, L.sp.heads, L.sp.vdim, tl_swa_splits(T, L.sp.window, st->cfg.max_positions));
+        ws = n > ws ? n : ws;
+      }
+    TL_TRY(dev_alloc(st, &st->swa_ws, ws));
+  }
   if (st->max_top) {
     const size_t S = C * st->max_top;
     TL_TRY(dev_alloc(st, &st->ids, S));
@@ -526,6 +536,8 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
     a.scale = sp.scale;
     a.start_pos = start_pos;
     a.pos_dev = pos_dev;
+    a.nsplit = tl_swa_splits(T, sp.window, c.max_positions);
+    a.ws = st->swa_ws;
     TL_TRY(tl_launch_swa(a, s));
     TL_TRY(project(st, L.wo, W, L.od, st->att, L.od, st->proj, W, T, s));
     ResidNormArgs n = {};

@@ -8,6 +8,7 @@
 // are accumulated with the lanes spread over the value columns (coalesced rows of V; a key's weight is read from its lane). The four waves' partial
 // (max, sum, output) are merged through LDS at the end.
 #include <math.h>
+#include <stdlib.h>
 
 #include "tl_stack.h"
 
@@ -37,7 +38,12 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
 #pragma unroll
   for (int r = 0; r < SWA_MAX_VR; ++r) o[r] = 0.0f;
   const int pieces = (n + 63) >> 6;
-  for (int c = wave; c < pieces; c += SWA_WAVES) {
+  // nsplit > 1 (few tokens, long windows): workgroup z of (token, head) takes pieces [z * per, (z + 1) * per) and leaves its
+  // (max, sum, unnormalised output) in ws for swa_combine_kernel
+  const int nsplit = a.nsplit > 1 ? a.nsplit : 1;
+  const int per = (pieces + nsplit - 1) / nsplit;
+  const int c_lo = blockIdx.z * per, c_hi = c_lo + per < pieces ? c_lo + per : pieces;
+  for (int c = c_lo + wave; c < c_hi; c += SWA_WAVES) {
     const int j0 = jlo + c * 64;
     const int j = j0 + lane;
     const bool valid = j <= i;
@@ -71,7 +77,25 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
 #pragma unroll
     for (int r = 0; r < SWA_MAX_VR; ++r) o[r] *= corr;
     const float* vp = a.vc + (size_t)j0 * vld + (size_t)g * a.vdim;
-    for (int jj = 0; jj < cnt; ++jj) {  // jj is wave-uniform: the weight of key jj comes straight from its lane's register
+    // jj is wave-uniform: the weight of key jj comes straight from its lane's register; four rows of V per step, so that
+    // their loads are in flight together
+    int jj = 0;
+    for (; jj + 4 <= cnt; jj += 4) {
+      const float p0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj));
+      const float p1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + 1));
+      const float p2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + 2));
+      const float p3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + 3));
+      const float* vr = vp + (size_t)jj * vld;
+#pragma unroll
+      for (int r = 0; r < SWA_MAX_VR; ++r) {
+        const int d = lane + 64 * r;
+        if (d < a.vdim) {
+          const float v0 = vr[d], v1 = vr[vld + d], v2 = vr[2 * (size_t)vld + d], v3 = vr[3 * (size_t)vld + d];
+          o[r] += (p0 * v0 + p1 * v1) + (p2 * v2 + p3 * v3);
+        }
+      }
+    }
+    for (; jj < cnt; ++jj) {
       const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj));
       const float* vr = vp + (size_t)jj * vld;
 #pragma unroll
@@ -97,8 +121,22 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   float f[SWA_WAVES], L = 0.0f;
 #pragma unroll
   for (int w = 0; w < SWA_WAVES; ++w) {
-    f[w] = expf(ml[w * 2] - M);  // a wave without a piece: exp(-inf) = 0
+    f[w] = ml[w * 2] == -INFINITY ? 0.0f : expf(ml[w * 2] - M);  // a wave without a piece counts nothing
     L += ml[w * 2 + 1] * f[w];
+  }
+  if (nsplit > 1) {
+    float* rec = a.ws + (((size_t)t * a.heads + h) * nsplit + blockIdx.z) * (a.vdim + 2);
+    if (tid == 0) {
+      rec[0] = M;  // -inf and sum 0 when this split had no piece
+      rec[1] = M == -INFINITY ? 0.0f : L;
+    }
+    for (int d = tid; d < a.vdim; d += 256) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int w = 0; w < SWA_WAVES; ++w) acc += f[w] == 0.0f ? 0.0f : ow[w * a.vdim + d] * f[w];
+      rec[2 + d] = M == -INFINITY ? 0.0f : acc;
+    }
+    return;
   }
   float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
   for (int d = tid; d < a.vdim; d += 256) {
@@ -109,7 +147,269 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   }
 }
 
+// out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M) over the nsplit records of a (token, head), in split order
+__global__ __launch_bounds__(64) void swa_combine_kernel(const SwaArgs a) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int rs = a.vdim + 2;
+  const float* rec = a.ws + ((size_t)t * a.heads + h) * a.nsplit * rs;
+  // lane z holds record z's max and sum (nsplit <= 64): one round trip, then everything is in registers
+  const float mz = lane < a.nsplit ? rec[(size_t)lane * rs] : -INFINITY;
+  const float lz = lane < a.nsplit ? rec[(size_t)lane * rs + 1] : 0.0f;
+  float M = mz;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  const float fz = mz == -INFINITY ? 0.0f : expf(mz - M);
+  float L = 0.0f;
+  for (int z = 0; z < a.nsplit; ++z) L += __shfl(lz * fz, z);  // in split order
+  float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
+  for (int d0 = 0; d0 < a.vdim; d0 += 64) {  // every lane stays in the loop: a shuffle reads nothing from a lane that has left
+    const int d = d0 + lane;
+    float acc = 0.0f;
+    for (int z = 0; z < a.nsplit; ++z) {
+      const float f = __shfl(fz, z);
+      if (d < a.vdim) acc += rec[(size_t)z * rs + 2 + d] * f;
+    }
+    if (d < a.vdim) op[d] = acc / L;
+  }
+}
+
+// ---- prompt chunks on the FP32 matrix instruction (v_mfma_f32_32x32x2_f32: exact FP32 products, FP32 accumulation) --------
+// One workgroup of 4 waves per (32-query tile, head). The key tiles of 32 positions that any query of the tile can see
+// (from the first query's window start to the last query's position) are dealt round-robin to the waves; each wave walks its
+// tiles with an online softmax of its own and the four (max, sum, O) are merged through LDS in wave order.
+//   S^T[key][query] = K Q^T: A = a lane's own cache row (16 bytes per load: lane half h owns d = 8 i + 4 h + 0..3 -- the
+//     order of a sum does not matter to the instruction), B = the query tile in LDS, zero-padded to a multiple of 8.
+//   The result has the query on the lane and 16 keys in registers; those registers are the A operand of O += P V as they
+//     stand (the result layout puts the key index where the next product's k index lives); V rows are read 128 B per half wave.
+typedef float swa_f32x4 __attribute__((ext_vector_type(4)));
+typedef float swa_f32x16 __attribute__((ext_vector_type(16)));
+
+// key (row of the 32x32 result) held in accumulator register e of lane half h
+__device__ __forceinline__ int swa_acc_row(int e, int h) { return (e & 3) + 8 * (e >> 2) + 4 * h; }
+
+__host__ __device__ inline int swa_dim_padded(int dim) { return (dim + 7) & ~7; }
+constexpr int SWA_SLOTS = 2;     // output slots in LDS: waves w and w + 2 share slot w (added in wave order)
+constexpr int SWA_KREG4 = 16;    // 16-byte pieces of a key row a lane half can hold in registers: dim <= 128
+__host__ __device__ inline size_t swa_mfma_lds_floats(int dim, int db) {
+  return (size_t)32 * (swa_dim_padded(dim) + 4) + 3 * SWA_WAVES * 32 + 32 + (size_t)SWA_SLOTS * 32 * 32 * db;
+}
+
+// DB: value columns per lane (vdim <= 32 * DB; lane r owns columns DB * r .. DB * r + DB - 1, one wide load per V row).
+// PRE: the lane's key row lives in registers (dim <= 128) and the NEXT tile's row is asked for as soon as the products have
+// read this one, so that its round trip runs under the softmax and P V of the tile in hand.
+template <int DB, bool PRE>
+__global__ __launch_bounds__(256) void swa_mfma_kernel(const SwaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dp = swa_dim_padded(a.dim), qs = dp + 4, dk = dp / 8;
+  float* sm_q = lds;                        // [32][dp + 4]
+  float* sm_m = sm_q + 32 * qs;             // [waves][32] running max per query
+  float* sm_l = sm_m + SWA_WAVES * 32;      // [waves][32] sum
+  float* sm_f = sm_l + SWA_WAVES * 32;      // [waves][32] the wave's factor exp(m_w - M)
+  float* sm_inv = sm_f + SWA_WAVES * 32;    // [32] 1 / L
+  float* sm_o = sm_inv + 32;                // [slots][32][32 * DB]
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, h = lane >> 5, wave = tid >> 6;
+  const int head = blockIdx.y, q0 = blockIdx.x * 32;
+  const int g = head / (a.heads / a.kv_heads);
+  const int start = a.pos_dev ? *a.pos_dev : a.start_pos;
+  const int kld = a.kv_heads * a.dim, vld = a.kv_heads * a.vdim;
+  const int last_i = q0 + 31 < a.T ? q0 + 31 : a.T - 1;
+  const int qpos = start + (q0 + r < a.T ? q0 + r : a.T - 1);  // rows beyond the chunk repeat its last query; never stored
+  const int last_q = start + last_i;
+  const int klo = a.window > 0 && start + q0 - a.window + 1 > 0 ? start + q0 - a.window + 1 : 0;
+  const int t_lo = klo >> 5, t_hi = last_q >> 5;
+  const bool kvec = (a.dim & 3) == 0 && ((size_t)a.kc & 15) == 0;
+  const bool vvec = (a.vdim % DB) == 0 && (DB == 1 || (((size_t)a.vc & 15) == 0 && (DB != 3)));
+  // piece i (d = 8 i + 4 h + 0..3) of the lane's key row of a tile; rows outside [klo, last_q] are seen by no query of the
+  // tile (masked below): their loads stay inside that range, so that nothing is read that the tile could not read
+  auto load_k4 = [&](int tile, int i) -> swa_f32x4 {
+    const int pr = tile * 32 + r;
+    const int krow = pr > last_q ? last_q : pr < klo ? klo : pr;
+    const float* kp = a.kc + (size_t)krow * kld + (size_t)g * a.dim + 4 * h + 8 * i;
+    const int d = 8 * i + 4 * h;
+    swa_f32x4 kv;
+    if (kvec) {
+      kv = d + 4 <= a.dim ? *reinterpret_cast<const swa_f32x4*>(kp) : swa_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) kv[c] = d + c < a.dim ? kp[c] : 0.0f;
+    }
+    return kv;
+  };
+  swa_f32x4 kreg[PRE ? SWA_KREG4 : 1];
+  if (PRE && t_lo + wave <= t_hi) {
+#pragma unroll
+    for (int i = 0; i < SWA_KREG4; ++i)
+      if (i < dk) kreg[i] = load_k4(t_lo + wave, i);
+  }
+  for (int i = tid; i < 32 * dp; i += 256) {
+    const int row = i / dp, d = i - row * dp;
+    sm_q[row * qs + d] = (q0 + row < a.T && d < a.dim) ? a.q[(size_t)(q0 + row) * a.ldq + (size_t)head * a.dim + d] : 0.0f;
+  }
+  __syncthreads();
+  swa_f32x16 o[DB];
+#pragma unroll
+  for (int b = 0; b < DB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[b][e] = 0.0f;
+  float mrun = -INFINITY, lrun = 0.0f;
+  const float* qrow = sm_q + r * qs + 4 * h;
+  for (int tile = t_lo + wave; tile <= t_hi; tile += SWA_WAVES) {
+    const int p0 = tile * 32;
+    swa_f32x16 s;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+    if (PRE) {
+#pragma unroll
+      for (int i = 0; i < SWA_KREG4; ++i)
+        if (i < dk) {
+          const swa_f32x4 qv = *reinterpret_cast<const swa_f32x4*>(qrow + 8 * i);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i][c], qv[c], s, 0, 0, 0);
+        }
+      if (tile + SWA_WAVES <= t_hi) {
+#pragma unroll
+        for (int i = 0; i < SWA_KREG4; ++i)
+          if (i < dk) kreg[i] = load_k4(tile + SWA_WAVES, i);
+      }
+    } else {
+      for (int i = 0; i < dk; ++i) {
+        const swa_f32x4 kv = load_k4(tile, i);
+        const swa_f32x4 qv = *reinterpret_cast<const swa_f32x4*>(qrow + 8 * i);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[c], qv[c], s, 0, 0, 0);
+      }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int p = p0 + swa_acc_row(e, h);
+      const bool seen = p <= qpos && (a.window <= 0 || qpos - p < a.window);
+      s[e] = seen ? s[e] * a.scale : -INFINITY;
+      tmax = fmaxf(tmax, s[e]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+    const float mnew = fmaxf(mrun, tmax);  // may still be -inf: a tile can lie wholly outside one query's window
+    const float corr = mrun == -INFINITY ? 0.0f : expf(mrun - mnew);
+    mrun = mnew;
+    float psum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s[e] = s[e] == -INFINITY ? 0.0f : expf(s[e] - mnew);
+      psum += s[e];
+    }
+    lrun = lrun * corr + psum;
+    if (__any(corr != 1.0f)) {  // O's rows are queries: each row's factor comes from the lane that owns the query
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float c = __shfl(corr, swa_acc_row(e, h));
+#pragma unroll
+        for (int b = 0; b < DB; ++b) o[b][e] *= c;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      int vrow = p0 + swa_acc_row(e, h);
+      vrow = vrow > last_q ? last_q : vrow < klo ? klo : vrow;  // masked keys carry weight 0
+      const float* vp = a.vc + (size_t)vrow * vld + (size_t)g * a.vdim + DB * r;
+      float vv[DB];
+      if (vvec && DB * r < a.vdim) {
+        if (DB == 4) {
+          const swa_f32x4 t4 = *reinterpret_cast<const swa_f32x4*>(vp);
+#pragma unroll
+          for (int b = 0; b < DB; ++b) vv[b] = t4[b];
+        } else if (DB == 2) {
+          const float2 t2 = *reinterpret_cast<const float2*>(vp);
+          vv[0] = t2.x;
+          vv[DB - 1] = t2.y;
+        } else {
+#pragma unroll
+          for (int b = 0; b < DB; ++b) vv[b] = vp[b];
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < DB; ++b) vv[b] = DB * r + b < a.vdim ? vp[b] : 0.0f;
+      }
+#pragma unroll
+      for (int b = 0; b < DB; ++b) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[e], vv[b], o[b], 0, 0, 0);
+    }
+  }
+  const float ltot = lrun + __shfl_xor(lrun, 32);
+  if (h == 0) {
+    sm_m[wave * 32 + r] = mrun;
+    sm_l[wave * 32 + r] = ltot;
+  }
+  __syncthreads();
+  if (h == 0) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < SWA_WAVES; ++w) M = fmaxf(M, sm_m[w * 32 + r]);  // finite: every query sees itself
+    const float mw = sm_m[wave * 32 + r];
+    sm_f[wave * 32 + r] = mw == -INFINITY ? 0.0f : expf(mw - M);
+    if (wave == 0) {
+      float L = 0.0f;
+#pragma unroll
+      for (int w = 0; w < SWA_WAVES; ++w) {
+        const float m2 = sm_m[w * 32 + r];
+        L += m2 == -INFINITY ? 0.0f : sm_l[w * 32 + r] * expf(m2 - M);
+      }
+      sm_inv[r] = 1.0f / L;
+    }
+  }
+  __syncthreads();
+  // merge in wave order through SWA_SLOTS slots: waves 0, 1 store, then waves 2, 3 add to the slot of wave - 2
+  constexpr int OW = 32 * DB;
+  float* slot = sm_o + (size_t)(wave % SWA_SLOTS) * 32 * OW;
+#pragma unroll
+  for (int round = 0; round < SWA_WAVES / SWA_SLOTS; ++round) {
+    if (wave / SWA_SLOTS == round) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = swa_acc_row(e, h);
+        const float f = sm_f[wave * 32 + row];
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+          float* p = slot + row * OW + DB * r + b;
+          *p = round == 0 ? o[b][e] * f : *p + o[b][e] * f;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int i = tid; i < 32 * OW; i += 256) {
+    const int row = i / OW, col = i - row * OW;
+    if (q0 + row >= a.T || col >= a.vdim) continue;
+    float acc = 0.0f;
+#pragma unroll
+    for (int w = 0; w < SWA_SLOTS; ++w) acc += sm_o[(size_t)w * 32 * OW + i];
+    a.out[(size_t)(q0 + row) * a.heads * a.vdim + (size_t)head * a.vdim + col] = acc * sm_inv[row];
+  }
+}
+
+template <int DB, bool PRE>
+int launch_swa_mfma_as(const SwaArgs& a, hipStream_t s) {
+  static TlDeviceOnce lds_raised;  // per instantiation, per device
+  const size_t lds = sizeof(float) * swa_mfma_lds_floats(a.dim, DB);
+  TL_TRY(tl_raise_lds_limit(swa_mfma_kernel<DB, PRE>, 160 * 1024, lds_raised));
+  swa_mfma_kernel<DB, PRE><<<dim3((a.T + 31) / 32, a.heads), 256, lds, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+template <int DB>
+int launch_swa_mfma(const SwaArgs& a, hipStream_t s) {
+  return swa_dim_padded(a.dim) <= 8 * SWA_KREG4 ? launch_swa_mfma_as<DB, true>(a, s) : launch_swa_mfma_as<DB, false>(a, s);
+}
+
 }  // namespace
+
+// prompt chunks whose shapes fit go to the matrix cores (TL_SWA_MFMA=0: never)
+static bool swa_mfma_wanted(const SwaArgs& a) {
+  static const bool on = [] {
+    const char* e = getenv("TL_SWA_MFMA");
+    return !e || atoi(e) != 0;
+  }();
+  const int db = (a.vdim + 31) / 32;
+  return on && a.T >= 16 && db <= 4 && sizeof(float) * swa_mfma_lds_floats(a.dim, db) <= 160 * 1024;
+}
 
 int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
   TL_REQUIRE(a.q && a.kc && a.vc && a.out && a.T > 0, "swa: bad arguments");
@@ -118,13 +418,36 @@ int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
   TL_REQUIRE(a.dim > 0 && a.vdim > 0 && a.vdim <= 64 * SWA_MAX_VR, "swa: value size %d outside (0, %d]", a.vdim,
              64 * SWA_MAX_VR);
   TL_REQUIRE(a.pos_dev || a.start_pos >= 0, "swa: negative start position");
+  TL_REQUIRE(a.heads <= 65535, "swa: too many heads");
+  if (swa_mfma_wanted(a)) {
+    switch ((a.vdim + 31) / 32) {
+      case 1: return launch_swa_mfma<1>(a, s);
+      case 2: return launch_swa_mfma<2>(a, s);
+      case 3: return launch_swa_mfma<3>(a, s);
+      default: return launch_swa_mfma<4>(a, s);
+    }
+  }
   const size_t lds = sizeof(float) * (((a.dim + 3) & ~3) + SWA_WAVES * a.vdim + SWA_WAVES * 2);
   TL_REQUIRE(lds <= 64 * 1024, "swa: key size %d too large", a.dim);
   TL_REQUIRE(a.heads <= 65535, "swa: too many heads");
-  swa_kernel<<<dim3(a.T, a.heads), 256, lds, s>>>(a);
+  const int nsplit = a.nsplit > 1 ? a.nsplit : 1;
+  TL_REQUIRE(nsplit == 1 || a.ws, "swa: split launch without a workspace");
+  TL_REQUIRE(nsplit <= 64, "swa: %d splits", nsplit);
+  swa_kernel<<<dim3(a.T, a.heads, nsplit), 256, lds, s>>>(a);
+  if (nsplit > 1) swa_combine_kernel<<<dim3(a.T, a.heads), 64, 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }
+
+int tl_swa_splits(int T, int window, int max_pos) {
+  if (T > 4) return 1;  // a chunk of a prompt has workgroups enough
+  const int keys = window > 0 && window < max_pos ? window : max_pos;
+  const int pieces = (keys + 63) / 64;
+  int n = (pieces + SWA_WAVES - 1) / SWA_WAVES;  // a piece per wave and split
+  return n < 1 ? 1 : n > 32 ? 32 : n;
+}
+
+size_t tl_swa_ws_floats(int T, int heads, int vdim, int nsplit) { return (size_t)T * heads * nsplit * (vdim + 2); }
 
 extern "C" int tl_swa_attention(const float* q_dev, const float* k_cache_dev, const float* v_cache_dev, float* out_dev,
                                 int num_tokens, int start_pos, int heads, int kv_heads, int dim, int vdim, int window,
@@ -143,5 +466,11 @@ extern "C" int tl_swa_attention(const float* q_dev, const float* k_cache_dev, co
   a.window = window;
   a.scale = scale;
   a.start_pos = start_pos;
+  a.nsplit = tl_swa_splits(num_tokens, window, start_pos + num_tokens);
+  if (a.nsplit > 1) {
+    void* ws = nullptr;
+    TL_TRY(tl_scratch(TL_SCRATCH_ATTN, sizeof(float) * tl_swa_ws_floats(num_tokens, heads, vdim, a.nsplit), &ws));
+    a.ws = static_cast<float*>(ws);
+  }
   return tl_launch_swa(a, static_cast<hipStream_t>(stream));
 }
