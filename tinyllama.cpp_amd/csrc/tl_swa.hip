@@ -198,7 +198,7 @@ __host__ __device__ inline size_t swa_mfma_lds_floats(int dim, int db) {
 // PRE: the lane's key row lives in registers (dim <= 128) and the NEXT tile's row is asked for as soon as the products have
 // read this one, so that its round trip runs under the softmax and P V of the tile in hand.
 template <int DB, bool PRE>
-__global__ __launch_bounds__(256) void swa_mfma_kernel(const SwaArgs a) {
+__global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  // two workgroups per CU: 256 registers a lane
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int dp = swa_dim_padded(a.dim), qs = dp + 4, dk = dp / 8;
   float* sm_q = lds;                        // [32][dp + 4]
@@ -234,6 +234,33 @@ __global__ __launch_bounds__(256) void swa_mfma_kernel(const SwaArgs a) {
       for (int c = 0; c < 4; ++c) kv[c] = d + c < a.dim ? kp[c] : 0.0f;
     }
     return kv;
+  };
+  // the lane's DB value columns of the keys held in accumulator registers e0 .. e0 + 7 (masked keys carry weight 0; their
+  // rows are clamped like the key rows)
+  auto load_v = [&](int p0, int e0, float (*vv)[DB]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      int vrow = p0 + swa_acc_row(e0 + e, h);
+      vrow = vrow > last_q ? last_q : vrow < klo ? klo : vrow;
+      const float* vp = a.vc + (size_t)vrow * vld + (size_t)g * a.vdim + DB * r;
+      if (vvec && DB * r < a.vdim) {
+        if (DB == 4) {
+          const swa_f32x4 t4 = *reinterpret_cast<const swa_f32x4*>(vp);
+#pragma unroll
+          for (int b = 0; b < DB; ++b) vv[e][b] = t4[b];
+        } else if (DB == 2) {
+          const float2 t2 = *reinterpret_cast<const float2*>(vp);
+          vv[e][0] = t2.x;
+          vv[e][DB - 1] = t2.y;
+        } else {
+#pragma unroll
+          for (int b = 0; b < DB; ++b) vv[e][b] = vp[b];
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < DB; ++b) vv[e][b] = DB * r + b < a.vdim ? vp[b] : 0.0f;
+      }
+    }
   };
   swa_f32x4 kreg[PRE ? SWA_KREG4 : 1];
   if (PRE && t_lo + wave <= t_hi) {
@@ -279,6 +306,8 @@ __global__ __launch_bounds__(256) void swa_mfma_kernel(const SwaArgs a) {
         for (int c = 0; c < 4; ++c) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[c], qv[c], s, 0, 0, 0);
       }
     }
+    float va[8][DB];
+    load_v(p0, 0, va);  // the V rows of the first 8 registers' keys: asked for now, needed after the softmax
     float tmax = -INFINITY;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
@@ -306,32 +335,16 @@ __global__ __launch_bounds__(256) void swa_mfma_kernel(const SwaArgs a) {
         for (int b = 0; b < DB; ++b) o[b][e] *= c;
       }
     }
+    float vb[8][DB];
+    load_v(p0, 8, vb);  // the second half's round trip runs under the first half's products
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      int vrow = p0 + swa_acc_row(e, h);
-      vrow = vrow > last_q ? last_q : vrow < klo ? klo : vrow;  // masked keys carry weight 0
-      const float* vp = a.vc + (size_t)vrow * vld + (size_t)g * a.vdim + DB * r;
-      float vv[DB];
-      if (vvec && DB * r < a.vdim) {
-        if (DB == 4) {
-          const swa_f32x4 t4 = *reinterpret_cast<const swa_f32x4*>(vp);
+    for (int e = 0; e < 8; ++e)
 #pragma unroll
-          for (int b = 0; b < DB; ++b) vv[b] = t4[b];
-        } else if (DB == 2) {
-          const float2 t2 = *reinterpret_cast<const float2*>(vp);
-          vv[0] = t2.x;
-          vv[DB - 1] = t2.y;
-        } else {
+      for (int b = 0; b < DB; ++b) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[e], va[e][b], o[b], 0, 0, 0);
 #pragma unroll
-          for (int b = 0; b < DB; ++b) vv[b] = vp[b];
-        }
-      } else {
+    for (int e = 0; e < 8; ++e)
 #pragma unroll
-        for (int b = 0; b < DB; ++b) vv[b] = DB * r + b < a.vdim ? vp[b] : 0.0f;
-      }
-#pragma unroll
-      for (int b = 0; b < DB; ++b) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[e], vv[b], o[b], 0, 0, 0);
-    }
+      for (int b = 0; b < DB; ++b) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[8 + e], vb[e][b], o[b], 0, 0, 0);
   }
   const float ltot = lrun + __shfl_xor(lrun, 32);
   if (h == 0) {
