@@ -72,7 +72,7 @@ def dev(env, a):
     return env["engine"].DeviceBuffer.from_numpy(np.ascontiguousarray(a))
 
 
-@pytest.mark.parametrize("rows,cols,T", [(64, 64, 64), (70, 40, 3), (129, 72, 130), (33, 37, 65), (256, 512, 200)])
+@pytest.mark.parametrize("rows,cols,T", [(64, 64, 64), (70, 40, 3), (129, 72, 130), (33, 37, 65), (256, 512, 200), (330, 100, 259)])
 def test_dense_matmul(env, rows, cols, T):
     synth, capi = env["synth"], env["capi"]
     rng = np.random.default_rng(rows + cols + T)
@@ -81,8 +81,15 @@ def test_dense_matmul(env, rows, cols, T):
     wd, xd = dev(env, w), dev(env, x)
     yd = env["engine"].DeviceBuffer(4 * T * rows)
     wf = synth.from_bf16(w).astype(np.float64)
-    for terms in (3, 1):
-        capi.check(capi.lib().tl_dense_matmul(wd.ptr, rows, cols, xd.ptr, yd.ptr, T, terms, None), "tl_dense_matmul")
+    for terms, tile in ((3, "64"), (1, "64"), (3, "128"), (1, "128"), (3, None)):  # both tile shapes, then the launcher's pick
+        if tile is None:
+            os.environ.pop("TL_DENSE_TILE", None)
+        else:
+            os.environ["TL_DENSE_TILE"] = tile
+        try:
+            capi.check(capi.lib().tl_dense_matmul(wd.ptr, rows, cols, xd.ptr, yd.ptr, T, terms, None), "tl_dense_matmul")
+        finally:
+            os.environ.pop("TL_DENSE_TILE", None)
         capi.check(capi.lib().tl_device_sync(), "sync")
         got = yd.to_numpy(np.float32, (T, rows))
         xin = x if terms == 3 else synth.from_bf16(synth.to_bf16(x))  # terms 1: exactly the bf16-rounded activations

@@ -8,9 +8,12 @@
 //   LDS: terms = 1 keeps their bf16 rounding, terms = 3 keeps hi + mid + lo (3 x 8 mantissa bits = all 24 of an FP32
 //   value); the weights are bf16 to begin with, so three MFMAs per product reproduce the FP32 product exactly and only the
 //   order of the FP32 accumulation differs from a scalar loop.
-//   A workgroup of 4 waves owns a 64-feature x 64-token tile, BK = 32. Items may be gathered (x_rows), scattered (y_rows) and
+//   A workgroup of 4 waves owns a 64 x 64 or (enough rows and tokens) a 128 x 128 feature x token tile, BK = 32, with the
+//   next k-block's global loads in flight under the products of the block in LDS. Items may be gathered (x_rows), scattered (y_rows) and
 //   grouped (group_off: blockIdx.z = matrix of the group; tiles beyond a group's items leave at once), which is what the
 //   experts of a mixture need: the plan lives on the device, the grid is sized for the worst case.
+#include <stdlib.h>
+
 #include "tl_bf16.h"
 #include "tl_stack.h"
 
@@ -26,10 +29,13 @@ __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest e
 }
 __device__ __forceinline__ float bf2f(unsigned short h) { return tl_bf2f(h); }
 
-constexpr int BM = 64, BN = 64, BK = 32, LDK = 40;  // LDK: padded row of a tile in LDS (80 B, keeps 16 B / 8 B alignment)
+constexpr int BK = 32, LDK = 40;  // LDK: padded row of a tile in LDS (80 B, keeps 16 B / 8 B alignment)
 
-template <int TERMS>
+// A workgroup of 4 waves (2 x 2) owns a (64 WM)-feature x (64 WN)-token tile; a wave WM x WN products of 32 x 32. The next
+// k-block's weights and activations are asked for (into registers) before the products of the block in LDS start.
+template <int TERMS, int WM, int WN>
 __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
   __shared__ __attribute__((aligned(16))) unsigned short Ws[BM][LDK];
   __shared__ __attribute__((aligned(16))) unsigned short Xs[TERMS][BN][LDK];
   __shared__ int xrow[BN];
@@ -43,94 +49,132 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
   if (t0 >= hi) return;
   const int f0 = blockIdx.x * BM;
   const unsigned short* W = a.w + (size_t)g * a.rows * a.cols;
-  if (tid < BN) {
-    const int it = t0 + tid;
+  for (int i = tid; i < BN; i += 256) {
+    const int it = t0 + i;
     int r = -1;
     if (it < hi) r = a.x_rows ? a.x_rows[it] / a.x_div : it;
-    xrow[tid] = r;
+    xrow[i] = r;
   }
   __syncthreads();
   const int wave = tid >> 6, lane = tid & 63, wm = wave & 1, wn = wave >> 1;
-  const int lr = tid >> 2, lk = (tid & 3) * 8;  // this thread stages 8 consecutive k of row lr of both tiles
+  const int lr = tid >> 2, lk = (tid & 3) * 8;  // this thread stages 8 consecutive k of rows lr + 64 i of both tiles
   const int K = a.cols;
   const bool vec = (K & 7) == 0 && (a.ldx & 3) == 0 && ((size_t)a.x & 15) == 0 && ((size_t)W & 15) == 0;
-  const int frow = f0 + lr;
-  const int xr = xrow[lr];
-  const unsigned short* wp = W + (size_t)(frow < a.rows ? frow : 0) * K;
-  const float* xp = a.x + (size_t)(xr >= 0 ? xr : 0) * a.ldx;
-  f32x16 acc;
+  const unsigned short* wp[WM];
+  const float* xp[WN];
+  bool wok[WM], xok[WN];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-  for (int k0 = 0; k0 < K; k0 += BK) {
+  for (int i = 0; i < WM; ++i) {
+    const int frow = f0 + lr + 64 * i;
+    wok[i] = frow < a.rows;
+    wp[i] = W + (size_t)(wok[i] ? frow : 0) * K;
+  }
+#pragma unroll
+  for (int j = 0; j < WN; ++j) {
+    const int xr = xrow[lr + 64 * j];
+    xok[j] = xr >= 0;
+    xp[j] = a.x + (size_t)(xok[j] ? xr : 0) * a.ldx;
+  }
+  uint4 wreg[WM];
+  float xreg[WN][8];
+  auto fetch = [&](int k0) __attribute__((always_inline)) {
     const int k = k0 + lk;
-    unsigned short wv[8];
-    float xv[8];
     if (vec && k + 8 <= K) {
-      const uint4 w4 = frow < a.rows ? *reinterpret_cast<const uint4*>(wp + k) : make_uint4(0, 0, 0, 0);
-      wv[0] = w4.x & 0xffff; wv[1] = w4.x >> 16; wv[2] = w4.y & 0xffff; wv[3] = w4.y >> 16;
-      wv[4] = w4.z & 0xffff; wv[5] = w4.z >> 16; wv[6] = w4.w & 0xffff; wv[7] = w4.w >> 16;
-      float4 x0 = make_float4(0, 0, 0, 0), x1 = x0;
-      if (xr >= 0) {
-        x0 = *reinterpret_cast<const float4*>(xp + k);
-        x1 = *reinterpret_cast<const float4*>(xp + k + 4);
+#pragma unroll
+      for (int i = 0; i < WM; ++i) wreg[i] = wok[i] ? *reinterpret_cast<const uint4*>(wp[i] + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        float4 x0 = make_float4(0, 0, 0, 0), x1 = x0;
+        if (xok[j]) {
+          x0 = *reinterpret_cast<const float4*>(xp[j] + k);
+          x1 = *reinterpret_cast<const float4*>(xp[j] + k + 4);
+        }
+        xreg[j][0] = x0.x; xreg[j][1] = x0.y; xreg[j][2] = x0.z; xreg[j][3] = x0.w;
+        xreg[j][4] = x1.x; xreg[j][5] = x1.y; xreg[j][6] = x1.z; xreg[j][7] = x1.w;
       }
-      xv[0] = x0.x; xv[1] = x0.y; xv[2] = x0.z; xv[3] = x0.w;
-      xv[4] = x1.x; xv[5] = x1.y; xv[6] = x1.z; xv[7] = x1.w;
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const bool in = k + i < K;
-        wv[i] = (in && frow < a.rows) ? wp[k + i] : (unsigned short)0;
-        xv[i] = (in && xr >= 0) ? xp[k + i] : 0.0f;
-      }
-    }
-    {
-      uint4 p;
-      p.x = wv[0] | ((unsigned)wv[1] << 16); p.y = wv[2] | ((unsigned)wv[3] << 16);
-      p.z = wv[4] | ((unsigned)wv[5] << 16); p.w = wv[6] | ((unsigned)wv[7] << 16);
-      *reinterpret_cast<uint4*>(&Ws[lr][lk]) = p;
-    }
+      for (int i = 0; i < WM; ++i) {
+        unsigned short wv[8];
 #pragma unroll
-    for (int t = 0; t < TERMS; ++t) {
-      unsigned short h[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        h[i] = f2bf(xv[i]);
-        xv[i] -= bf2f(h[i]);  // exact: the remainder of an FP32 value after its leading 8 bits
+        for (int e = 0; e < 8; ++e) wv[e] = (k + e < K && wok[i]) ? wp[i][k + e] : (unsigned short)0;
+        wreg[i].x = wv[0] | ((unsigned)wv[1] << 16); wreg[i].y = wv[2] | ((unsigned)wv[3] << 16);
+        wreg[i].z = wv[4] | ((unsigned)wv[5] << 16); wreg[i].w = wv[6] | ((unsigned)wv[7] << 16);
       }
-      uint4 p;
-      p.x = h[0] | ((unsigned)h[1] << 16); p.y = h[2] | ((unsigned)h[3] << 16);
-      p.z = h[4] | ((unsigned)h[5] << 16); p.w = h[6] | ((unsigned)h[7] << 16);
-      *reinterpret_cast<uint4*>(&Xs[t][lr][lk]) = p;
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xreg[j][e] = (k + e < K && xok[j]) ? xp[j][k + e] : 0.0f;
+    }
+  };
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) *reinterpret_cast<uint4*>(&Ws[lr + 64 * i][lk]) = wreg[i];
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+#pragma unroll
+      for (int t = 0; t < TERMS; ++t) {
+        unsigned short h[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          h[e] = f2bf(xreg[j][e]);
+          xreg[j][e] -= bf2f(h[e]);  // exact: the remainder of an FP32 value after its leading 8 bits
+        }
+        uint4 p;
+        p.x = h[0] | ((unsigned)h[1] << 16); p.y = h[2] | ((unsigned)h[3] << 16);
+        p.z = h[4] | ((unsigned)h[5] << 16); p.w = h[6] | ((unsigned)h[7] << 16);
+        *reinterpret_cast<uint4*>(&Xs[t][lr + 64 * j][lk]) = p;
+      }
     }
     __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);  // in flight while the products below run
 #pragma unroll
     for (int ks = 0; ks < BK / 8; ++ks) {
       const int kk = ks * 8 + (lane >> 5) * 4;
-      const bf16x4 af = *reinterpret_cast<const bf16x4*>(&Ws[wm * 32 + (lane & 31)][kk]);
+      bf16x4 af[WM];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) af[i] = *reinterpret_cast<const bf16x4*>(&Ws[(wm * WM + i) * 32 + (lane & 31)][kk]);
 #pragma unroll
       for (int t = TERMS - 1; t >= 0; --t) {  // small terms first
-        const bf16x4 bfr = *reinterpret_cast<const bf16x4*>(&Xs[t][wn * 32 + (lane & 31)][kk]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(af, bfr, acc, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+          const bf16x4 bfr = *reinterpret_cast<const bf16x4*>(&Xs[t][(wn * WN + j) * 32 + (lane & 31)][kk]);
+#pragma unroll
+          for (int i = 0; i < WM; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(af[i], bfr, acc[i][j], 0, 0, 0);
+        }
       }
     }
     __syncthreads();
   }
-  // C layout: lane holds token (lane & 31) of its wave's 32, features (i / 4) * 8 + (lane >> 5) * 4 + (i & 3)
-  const int it = t0 + wn * 32 + (lane & 31);
-  if (it < hi) {
+  // C layout: lane holds token (lane & 31) of a 32 x 32 product, features (e / 4) * 8 + (lane >> 5) * 4 + (e & 3)
+  const bool v4 = (a.ldy & 3) == 0 && ((size_t)a.y & 15) == 0;
+#pragma unroll
+  for (int j = 0; j < WN; ++j) {
+    const int it = t0 + (wn * WN + j) * 32 + (lane & 31);
+    if (it >= hi) continue;
     const int orow = a.y_rows ? a.y_rows[it] : it;
     float* yr = a.y + (size_t)orow * a.ldy;
-    const bool v4 = (a.ldy & 3) == 0 && ((size_t)a.y & 15) == 0;
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const int f = f0 + wm * 32 + gq * 8 + (lane >> 5) * 4;
-      if (v4 && f + 4 <= a.rows) {
-        *reinterpret_cast<float4*>(yr + f) = make_float4(acc[gq * 4], acc[gq * 4 + 1], acc[gq * 4 + 2], acc[gq * 4 + 3]);
-      } else {
+    for (int i = 0; i < WM; ++i) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (f + i < a.rows) yr[f + i] = acc[gq * 4 + i];
+      for (int gq = 0; gq < 4; ++gq) {
+        const int f = f0 + (wm * WM + i) * 32 + gq * 8 + (lane >> 5) * 4;
+        if (v4 && f + 4 <= a.rows) {
+          *reinterpret_cast<float4*>(yr + f) =
+              make_float4(acc[i][j][gq * 4], acc[i][j][gq * 4 + 1], acc[i][j][gq * 4 + 2], acc[i][j][gq * 4 + 3]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (f + e < a.rows) yr[f + e] = acc[i][j][gq * 4 + e];
+        }
       }
     }
   }
@@ -160,10 +204,25 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
   TL_REQUIRE(!a.x_rows || a.x_div >= 1, "dense gemm: x_div must be >= 1");
   const int groups = a.groups > 0 ? a.groups : 1;
   TL_REQUIRE(groups == 1 || a.group_off, "dense gemm: groups without group_off");
+  // 128 x 128 tiles when there is enough of both sides to fill them (grouped launches: tokens per group on average)
+  const long long per_group = a.group_off ? (long long)a.T / groups : a.T;
+  // Measured at width 4096, chunks of 512 tokens: a dense launch has too few 128 x 128 tiles to fill 256 CUs (6144 x 512:
+  // 192 tiles, 117 us against 109 us in 768 small ones); the experts' grouped launches, whose small tiles are mostly
+  // half-empty, gain from them with one term (221 -> 193 us) and lose with three (356 -> 413 us).
+  const long long big_tiles = ((a.rows + 127) / 128) * ((per_group + 127) / 128) * groups;
+  const char* force = getenv("TL_DENSE_TILE");  // 64 / 128: tests and A/B runs pick the tile themselves
+  const bool big = force ? atoi(force) == 128
+                         : a.rows >= 256 && (a.group_off ? a.terms == 1 && per_group >= 96 : big_tiles >= 2 * tl_num_cus());
+  const int BM = big ? 128 : 64, BN = big ? 128 : 64;
   dim3 grid((a.rows + BM - 1) / BM, (a.T + BN - 1) / BN, groups);
   TL_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "dense gemm: launch too large");
-  if (a.terms == 1) dense_gemm_kernel<1><<<grid, 256, 0, s>>>(a);
-  else dense_gemm_kernel<3><<<grid, 256, 0, s>>>(a);
+  if (big) {
+    if (a.terms == 1) dense_gemm_kernel<1, 2, 2><<<grid, 256, 0, s>>>(a);
+    else dense_gemm_kernel<3, 2, 2><<<grid, 256, 0, s>>>(a);
+  } else {
+    if (a.terms == 1) dense_gemm_kernel<1, 1, 1><<<grid, 256, 0, s>>>(a);
+    else dense_gemm_kernel<3, 1, 1><<<grid, 256, 0, s>>>(a);
+  }
   TL_HIP(hipGetLastError());
   return 0;
 }
