@@ -48,6 +48,9 @@ struct SwaArgs {
   // (tl_swa_ws_floats floats) and are combined by a second small launch: the decode step's way to fill the chip
   int nsplit;
   float* ws;
+  // optional: T * heads zeroed counters (left at zero by every launch): the last workgroup of a (token, head) to arrive merges
+  // the records itself and the second launch falls away
+  unsigned* done_cnt;
 };
 int tl_launch_swa(const SwaArgs& a, hipStream_t s);
 int tl_swa_splits(int T, int window, int max_pos);  // splits worth having for T tokens over a cache of max_pos rows

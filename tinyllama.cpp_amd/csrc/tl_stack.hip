@@ -55,6 +55,7 @@ struct TlStack {
   float *gu_buf = nullptr, *act_buf = nullptr, *eout = nullptr, *sgu_buf = nullptr, *sact = nullptr, *sout = nullptr;
   float* wts = nullptr;
   float* swa_ws = nullptr;  // partial results of split attention launches (few tokens, long windows)
+  unsigned* swa_cnt = nullptr;  // their arrival counters (zero between launches)
   int *ids = nullptr, *off = nullptr, *slot_of = nullptr;
   int max_qkv = 0, max_od = 0, max_vd = 0, max_top = 0, max_experts = 0, max_gu = 0, max_sff = 0;
   tl_stack_layer_hook hook = nullptr;
@@ -313,6 +314,10 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
         ws = n > ws ? n : ws;
       }
     TL_TRY(dev_alloc(st, &st->swa_ws, ws));
+    size_t heads = 1;
+    for (const Layer& L : st->layers) heads = (size_t)L.sp.heads > heads ? (size_t)L.sp.heads : heads;
+    TL_TRY(dev_alloc(st, &st->swa_cnt, 4 * heads));
+    TL_HIP(hipMemsetAsync(st->swa_cnt, 0, sizeof(unsigned) * 4 * heads, s));
   }
   if (st->max_top) {
     const size_t S = C * st->max_top;
@@ -538,6 +543,7 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
     a.pos_dev = pos_dev;
     a.nsplit = tl_swa_splits(T, sp.window, c.max_positions);
     a.ws = st->swa_ws;
+    a.done_cnt = st->swa_cnt;
     TL_TRY(tl_launch_swa(a, s));
     TL_TRY(project(st, L.wo, W, L.od, st->att, L.od, st->proj, W, T, s));
     ResidNormArgs n = {};

@@ -17,6 +17,38 @@ namespace {
 constexpr int SWA_WAVES = 4;
 constexpr int SWA_MAX_VR = 4;  // value columns per lane: vdim <= 256
 
+__device__ __forceinline__ void swa_st_agent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float swa_ld_agent(const float* p) {  // past this CU's L1: the records come from other workgroups
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M) over the nsplit records of a (token, head), in split order; one wave
+__device__ __forceinline__ void swa_merge_records(const SwaArgs& a, int t, int h, int lane) {
+  const int rs = a.vdim + 2;
+  const float* rec = a.ws + ((size_t)t * a.heads + h) * a.nsplit * rs;
+  // lane z holds record z's max and sum (nsplit <= 64): one round trip, then everything is in registers
+  const float mz = lane < a.nsplit ? swa_ld_agent(rec + (size_t)lane * rs) : -INFINITY;
+  const float lz = lane < a.nsplit ? swa_ld_agent(rec + (size_t)lane * rs + 1) : 0.0f;
+  float M = mz;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  const float fz = mz == -INFINITY ? 0.0f : expf(mz - M);
+  float L = 0.0f;
+  for (int z = 0; z < a.nsplit; ++z) L += __shfl(lz * fz, z);  // in split order
+  float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
+  for (int d0 = 0; d0 < a.vdim; d0 += 64) {  // every lane stays in the loop: a shuffle reads nothing from a lane that has left
+    const int d = d0 + lane;
+    float acc = 0.0f;
+    for (int z = 0; z < a.nsplit; ++z) {
+      const float f = __shfl(fz, z);
+      if (d < a.vdim) acc += swa_ld_agent(rec + (size_t)z * rs + 2 + d) * f;
+    }
+    if (d < a.vdim) op[d] = acc / L;
+  }
+}
+
 __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   extern __shared__ float lds[];
   float* qs = lds;                                  // [dim]
@@ -52,7 +84,18 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
       const float* kp = a.kc + (size_t)j * kld + (size_t)g * a.dim;
       float acc = 0.0f;
       if (v4) {
-        for (int d = 0; d < a.dim; d += 4) {
+        int d = 0;
+        for (; d + 32 <= a.dim; d += 32) {  // eight 16-byte pieces of the key row in flight before the first product
+          float4 kv[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) kv[u] = *reinterpret_cast<const float4*>(kp + d + 4 * u);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const float4 qv = *reinterpret_cast<const float4*>(qs + d + 4 * u);
+            acc += qv.x * kv[u].x + qv.y * kv[u].y + qv.z * kv[u].z + qv.w * kv[u].w;
+          }
+        }
+        for (; d < a.dim; d += 4) {
           const float4 kv = *reinterpret_cast<const float4*>(kp + d);
           const float4 qv = *reinterpret_cast<const float4*>(qs + d);
           acc += qv.x * kv.x + qv.y * kv.y + qv.z * kv.z + qv.w * kv.w;
@@ -77,21 +120,23 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
 #pragma unroll
     for (int r = 0; r < SWA_MAX_VR; ++r) o[r] *= corr;
     const float* vp = a.vc + (size_t)j0 * vld + (size_t)g * a.vdim;
-    // jj is wave-uniform: the weight of key jj comes straight from its lane's register; four rows of V per step, so that
+    // jj is wave-uniform: the weight of key jj comes straight from its lane's register; eight rows of V per step, so that
     // their loads are in flight together
     int jj = 0;
-    for (; jj + 4 <= cnt; jj += 4) {
-      const float p0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj));
-      const float p1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + 1));
-      const float p2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + 2));
-      const float p3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + 3));
+    for (; jj + 8 <= cnt; jj += 8) {
+      float pj[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) pj[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), jj + u));
       const float* vr = vp + (size_t)jj * vld;
 #pragma unroll
       for (int r = 0; r < SWA_MAX_VR; ++r) {
         const int d = lane + 64 * r;
         if (d < a.vdim) {
-          const float v0 = vr[d], v1 = vr[vld + d], v2 = vr[2 * (size_t)vld + d], v3 = vr[3 * (size_t)vld + d];
-          o[r] += (p0 * v0 + p1 * v1) + (p2 * v2 + p3 * v3);
+          float vv[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) vv[u] = vr[(size_t)u * vld + d];
+          o[r] += ((pj[0] * vv[0] + pj[1] * vv[1]) + (pj[2] * vv[2] + pj[3] * vv[3])) +
+                  ((pj[4] * vv[4] + pj[5] * vv[5]) + (pj[6] * vv[6] + pj[7] * vv[7]));
         }
       }
     }
@@ -126,16 +171,32 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   }
   if (nsplit > 1) {
     float* rec = a.ws + (((size_t)t * a.heads + h) * nsplit + blockIdx.z) * (a.vdim + 2);
+    // (agent-scope stores: with the merge in this launch the reader may sit on another XCD, behind another L2)
     if (tid == 0) {
-      rec[0] = M;  // -inf and sum 0 when this split had no piece
-      rec[1] = M == -INFINITY ? 0.0f : L;
+      swa_st_agent(rec, M);  // -inf and sum 0 when this split had no piece
+      swa_st_agent(rec + 1, M == -INFINITY ? 0.0f : L);
     }
     for (int d = tid; d < a.vdim; d += 256) {
       float acc = 0.0f;
 #pragma unroll
       for (int w = 0; w < SWA_WAVES; ++w) acc += f[w] == 0.0f ? 0.0f : ow[w * a.vdim + d] * f[w];
-      rec[2 + d] = M == -INFINITY ? 0.0f : acc;
+      swa_st_agent(rec + 2 + d, M == -INFINITY ? 0.0f : acc);
     }
+    if (!a.done_cnt) return;  // swa_combine_kernel follows
+    // The last workgroup of this (token, head) to arrive merges the records itself (no second launch): the record stores
+    // are acknowledged, then one arrival per workgroup is counted; the counter goes back to zero for the next launch.
+    __shared__ int is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      unsigned* c = a.done_cnt + (size_t)t * a.heads + h;
+      const unsigned before = __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = before + 1u == (unsigned)nsplit;
+      if (is_last) __hip_atomic_store(c, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last || wave != 0) return;
+    swa_merge_records(a, t, h, lane);
     return;
   }
   float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
@@ -147,31 +208,7 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   }
 }
 
-// out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M) over the nsplit records of a (token, head), in split order
-__global__ __launch_bounds__(64) void swa_combine_kernel(const SwaArgs a) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int rs = a.vdim + 2;
-  const float* rec = a.ws + ((size_t)t * a.heads + h) * a.nsplit * rs;
-  // lane z holds record z's max and sum (nsplit <= 64): one round trip, then everything is in registers
-  const float mz = lane < a.nsplit ? rec[(size_t)lane * rs] : -INFINITY;
-  const float lz = lane < a.nsplit ? rec[(size_t)lane * rs + 1] : 0.0f;
-  float M = mz;
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
-  const float fz = mz == -INFINITY ? 0.0f : expf(mz - M);
-  float L = 0.0f;
-  for (int z = 0; z < a.nsplit; ++z) L += __shfl(lz * fz, z);  // in split order
-  float* op = a.out + (size_t)t * a.heads * a.vdim + (size_t)h * a.vdim;
-  for (int d0 = 0; d0 < a.vdim; d0 += 64) {  // every lane stays in the loop: a shuffle reads nothing from a lane that has left
-    const int d = d0 + lane;
-    float acc = 0.0f;
-    for (int z = 0; z < a.nsplit; ++z) {
-      const float f = __shfl(fz, z);
-      if (d < a.vdim) acc += rec[(size_t)z * rs + 2 + d] * f;
-    }
-    if (d < a.vdim) op[d] = acc / L;
-  }
-}
+__global__ __launch_bounds__(64) void swa_combine_kernel(const SwaArgs a) { swa_merge_records(a, blockIdx.x, blockIdx.y, threadIdx.x); }
 
 // ---- prompt chunks on the FP32 matrix instruction (v_mfma_f32_32x32x2_f32: exact FP32 products, FP32 accumulation) --------
 // One workgroup of 4 waves per (32-query tile, head). The key tiles of 32 positions that any query of the tile can see
@@ -447,7 +484,7 @@ int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
   TL_REQUIRE(nsplit == 1 || a.ws, "swa: split launch without a workspace");
   TL_REQUIRE(nsplit <= 64, "swa: %d splits", nsplit);
   swa_kernel<<<dim3(a.T, a.heads, nsplit), 256, lds, s>>>(a);
-  if (nsplit > 1) swa_combine_kernel<<<dim3(a.T, a.heads), 64, 0, s>>>(a);
+  if (nsplit > 1 && !a.done_cnt) swa_combine_kernel<<<dim3(a.T, a.heads), 64, 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }
