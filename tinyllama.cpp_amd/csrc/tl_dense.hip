@@ -12,6 +12,7 @@
 //   next k-block's global loads in flight under the products of the block in LDS. Items may be gathered (x_rows), scattered (y_rows) and
 //   grouped (group_off: blockIdx.z = matrix of the group; tiles beyond a group's items leave at once), which is what the
 //   experts of a mixture need: the plan lives on the device, the grid is sized for the worst case.
+#include <math.h>
 #include <stdlib.h>
 
 #include "tl_bf16.h"
@@ -28,6 +29,13 @@ __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest e
   return (unsigned short)(u >> 16);
 }
 __device__ __forceinline__ float bf2f(unsigned short h) { return tl_bf2f(h); }
+
+// y = g * sigmoid(alpha * g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit)  (tl_moe.hip has the operator)
+__device__ __forceinline__ float dense_glu(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+}
 
 constexpr int BK = 32, LDK = 40;  // LDK: padded row of a tile in LDS (80 B, keeps 16 B / 8 B alignment)
 
@@ -167,6 +175,13 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         const int f = f0 + (wm * WM + i) * 32 + gq * 8 + (lane >> 5) * 4;
+        if (a.glu) {  // (gate, up) pairs: features f, f + 1 -> unit f / 2; f + 2, f + 3 -> the next one
+#pragma unroll
+          for (int e = 0; e < 2; ++e)
+            if (f + 2 * e + 1 < a.rows)
+              yr[(f >> 1) + e] = dense_glu(acc[i][j][gq * 4 + 2 * e], acc[i][j][gq * 4 + 2 * e + 1], a.glu_limit, a.glu_alpha);
+          continue;
+        }
         if (v4 && f + 4 <= a.rows) {
           *reinterpret_cast<float4*>(yr + f) =
               make_float4(acc[i][j][gq * 4], acc[i][j][gq * 4 + 1], acc[i][j][gq * 4 + 2], acc[i][j][gq * 4 + 3]);
@@ -202,6 +217,7 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
   TL_REQUIRE(a.w && a.x && a.y && a.rows > 0 && a.cols > 0 && a.T > 0, "dense gemm: bad arguments");
   TL_REQUIRE(a.terms == 1 || a.terms == 3, "dense gemm: terms must be 1 or 3 (got %d)", a.terms);
   TL_REQUIRE(!a.x_rows || a.x_div >= 1, "dense gemm: x_div must be >= 1");
+  TL_REQUIRE(!a.glu || (a.rows & 1) == 0, "dense gemm: gated pairs need an even number of rows (got %d)", a.rows);
   const int groups = a.groups > 0 ? a.groups : 1;
   TL_REQUIRE(groups == 1 || a.group_off, "dense gemm: groups without group_off");
   // 128 x 128 tiles when there is enough of both sides to fill them (grouped launches: tokens per group on average)

@@ -938,6 +938,7 @@ extern "C" int tl_tp_local_group_decode(tl_model* const* ms, int n, int token_id
 extern "C" int tl_model_bench_kernel(tl_model* m, int kind, int iters, int warmup, float* avg_us_out,
                                      double* bytes_per_launch_out) {
   TL_REQUIRE(m && m->finalized && iters > 0 && warmup >= 0 && avg_us_out, "tl_model_bench_kernel: bad argument");
+  TL_REQUIRE(!m->stack, "tl_model_bench_kernel: the kinds are the Llama step's launches; a layer-list model has others");
   TL_REQUIRE(kind == 1 || kind == 4 || kind == 5 || kind == 6 || kind == 7 || kind == 9, "tl_model_bench_kernel: kind %d", kind);
   if (kind == 9) {  // the step's all-reduce of f32[hidden] (COLLECTIVE: every rank of the group makes the same call)
     TL_REQUIRE(m->tp > 1 && m->linked(), "tl_model_bench_kernel: kind 9 needs a linked tensor-parallel shard");

@@ -130,8 +130,8 @@ __global__ __launch_bounds__(256) void moe_decode_gu_kernel(const MoeDecodeArgs 
   const int ff = shared ? a.sff : a.ff;
   if (r >= ff) return;
   const unsigned short* gu = shared ? a.sgu : a.gu + (size_t)a.ids[j] * 2 * a.ff * a.width;
-  float gu2[2];  // row r of the gate and of the up matrix, their loads in flight together
-  tl_wave_dot_rows<2>(gu + (size_t)r * a.width, (size_t)ff * a.width, 2, a.x, a.width, vec != 0, lane, gu2);
+  float gu2[2];  // unit r's gate and up rows lie side by side; their loads are in flight together
+  tl_wave_dot_rows<2>(gu + (size_t)2 * r * a.width, (size_t)a.width, 2, a.x, a.width, vec != 0, lane, gu2);
   if (lane == 0) a.act[(size_t)j * a.ff + r] = glu_act(gu2[0], gu2[1], shared ? a.slimit : a.limit, a.alpha);
 }
 

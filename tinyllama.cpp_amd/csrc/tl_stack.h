@@ -27,6 +27,10 @@ struct DenseArgs {
   const int* y_rows;     // optional (device): item i writes output row y_rows[i]
   int groups;            // > 1 (or group_off set): group g uses matrix g and the items [group_off[g], group_off[g+1])
   const int* group_off;  // device, groups + 1 entries
+  // glu = 1: the rows are (gate, up) pairs -- row 2 i the gate, row 2 i + 1 the up projection of unit i -- and the epilogue
+  // stores the clamped gated unit of each pair instead of the pair: y[item][i] (ldy >= rows / 2), see tl_launch_glu_act
+  int glu;
+  float glu_limit, glu_alpha;
 };
 int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s);
 // y[rows] = W x for one token, FP32 throughout (weights widened exactly)
@@ -105,7 +109,8 @@ int tl_launch_moe_plan(const int* ids, int n_slots, int experts, int* off, int* 
 // out[p][i] = g * sigmoid(alpha * g) * (u + 1), g = min(in[p][i], limit), u = clamp(in[p][ff + i], -limit, limit)
 int tl_launch_glu_act(const float* in, int P, int ff, float limit, float alpha, float* out, hipStream_t s);
 // one token: the chosen experts' (and the shared expert's) gate/up GEMVs + activation, then the down GEMVs summed with the
-// router weights into y[width]. gu matrices are [2 * ff][width] (gate rows, then up rows), down [width][ff].
+// router weights into y[width]. gu matrices are [2 * ff][width] with row 2 i the gate and row 2 i + 1 the up projection of
+// unit i (the layout the chunk GEMM's fused activation wants); down [width][ff].
 struct MoeDecodeArgs {
   const float* x;        // [width]
   int width, top;

@@ -52,7 +52,7 @@ struct TlStack {
   bool gemv_decode = true;
   // workspaces for one chunk
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
-  float *gu_buf = nullptr, *act_buf = nullptr, *eout = nullptr, *sgu_buf = nullptr, *sact = nullptr, *sout = nullptr;
+  float *act_buf = nullptr, *eout = nullptr, *sact = nullptr, *sout = nullptr;
   float* wts = nullptr;
   float* swa_ws = nullptr;  // partial results of split attention launches (few tokens, long windows)
   unsigned* swa_cnt = nullptr;  // their arrival counters (zero between launches)
@@ -87,6 +87,13 @@ int upload_as_f32(float* dst, int type, const void* host, size_t n, hipStream_t 
     memcpy(wide.data(), host, n * 4);
   }
   TL_HIP(hipMemcpyAsync(dst, wide.data(), n * 4, hipMemcpyHostToDevice, s));
+  TL_HIP(hipStreamSynchronize(s));
+  return 0;
+}
+
+// rows of `cols` bf16 values to every second row of dst (gate rows to the even, up rows to the odd rows of a gate|up matrix)
+int upload_bf16_alternate(uint16_t* dst, const void* host, size_t rows, size_t cols, hipStream_t s) {
+  TL_HIP(hipMemcpy2DAsync(dst, 2 * cols * 2, host, cols * 2, cols * 2, rows, hipMemcpyHostToDevice, s));
   TL_HIP(hipStreamSynchronize(s));
   return 0;
 }
@@ -222,6 +229,13 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
                (long long)(c));                                                                                             \
     return upload_bf16((dst), host, (size_t)(r) * (size_t)(c), s);                                                          \
   } while (0)
+#define PAIRED(dst, r, c)                                                                                                   \
+  do {                                                                                                                      \
+    TL_REQUIRE(type == TL_BF16, "tl_stack_set_tensor: matrix %s must be bf16", name);                                       \
+    TL_REQUIRE(shape_is(shape, ndim, (r), (c)), "tl_stack_set_tensor: %s is not %lld x %lld", name, (long long)(r),         \
+               (long long)(c));                                                                                             \
+    return upload_bf16_alternate((dst), host, (size_t)(r), (size_t)(c), s);                                                 \
+  } while (0)
 #define VECTOR(dst, len)                                                                                                    \
   do {                                                                                                                      \
     TL_REQUIRE(shape_is(shape, ndim, (len)), "tl_stack_set_tensor: %s does not have %lld elements", name, (long long)(len)); \
@@ -264,22 +278,23 @@ int tl_stack_set_tensor(TlStack* st, const char* name, int type, const long long
     if (r == "mlp.router") MATRIX(L.router, sp.experts, W);
     if (r == "mlp.router.b") VECTOR(L.router_b, sp.experts);
     if (sff) {
-      if (r == "mlp.shared.gate") MATRIX(L.sgu, sff, W);
-      if (r == "mlp.shared.up") MATRIX(L.sgu + (size_t)sff * W, sff, W);
+      if (r == "mlp.shared.gate") PAIRED(L.sgu, sff, W);  // gate | up interleaved by unit (DenseArgs::glu)
+      if (r == "mlp.shared.up") PAIRED(L.sgu + W, sff, W);
       if (r == "mlp.shared.down") MATRIX(L.sdown, W, sff);
     }
     int e = -1, u2 = 0;
     if (sscanf(r.c_str(), "mlp.e%d.%n", &e, &u2) == 1 && u2 > 0 && e >= 0 && e < sp.experts) {
       const std::string k = r.substr(u2);
       uint16_t* gu = L.gu + (size_t)e * 2 * ff * W;
-      if (k == "gate") MATRIX(gu, ff, W);
-      if (k == "up") MATRIX(gu + (size_t)ff * W, ff, W);
+      if (k == "gate") PAIRED(gu, ff, W);
+      if (k == "up") PAIRED(gu + W, ff, W);
       if (k == "down") MATRIX(L.down + (size_t)e * W * ff, W, ff);
     }
   }
   --L.got;
   TL_REQUIRE(false, "tl_stack_set_tensor: no place for a tensor named %s in layer %d", name, li);
 #undef MATRIX
+#undef PAIRED
 #undef VECTOR
 }
 
@@ -325,11 +340,9 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
     TL_TRY(dev_alloc(st, &st->wts, S));
     TL_TRY(dev_alloc(st, &st->slot_of, S));
     TL_TRY(dev_alloc(st, &st->off, (size_t)st->max_experts + 1));
-    TL_TRY(dev_alloc(st, &st->gu_buf, C * st->max_gu));
     TL_TRY(dev_alloc(st, &st->act_buf, C * st->max_gu / 2 + st->max_sff));
     TL_TRY(dev_alloc(st, &st->eout, S * W));
     if (st->max_sff) {
-      TL_TRY(dev_alloc(st, &st->sgu_buf, C * 2 * st->max_sff));
       TL_TRY(dev_alloc(st, &st->sact, C * st->max_sff));
       TL_TRY(dev_alloc(st, &st->sout, C * W));
     }
@@ -455,16 +468,18 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
   g.cols = W;
   g.x = st->x;
   g.ldx = W;
-  g.y = st->gu_buf;
-  g.ldy = 2 * ff;
+  g.y = st->act_buf;  // the gated unit is applied in the epilogue: [S][ff]
+  g.ldy = ff;
   g.T = S;
   g.terms = terms_for(st, T);
   g.x_rows = st->slot_of;
   g.x_div = sp.top;
   g.groups = sp.experts;
   g.group_off = st->off;
+  g.glu = 1;
+  g.glu_limit = sp.expert_limit;
+  g.glu_alpha = sp.act_alpha;
   TL_TRY(tl_launch_dense_gemm(g, s));
-  TL_TRY(tl_launch_glu_act(st->gu_buf, S, ff, sp.expert_limit, sp.act_alpha, st->act_buf, s));
   DenseArgs d = {};  // down: item p writes the row of its slot, so that a token's choices lie side by side
   d.w = L.down;
   d.rows = W;
@@ -480,8 +495,20 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
   d.group_off = st->off;
   TL_TRY(tl_launch_dense_gemm(d, s));
   if (sff) {
-    TL_TRY(project(st, L.sgu, 2 * sff, W, st->x, W, st->sgu_buf, 2 * sff, T, s));
-    TL_TRY(tl_launch_glu_act(st->sgu_buf, T, sff, sp.shared_limit, sp.act_alpha, st->sact, s));
+    DenseArgs u = {};  // the shared expert's gate | up with the gated unit in the epilogue, then its down projection
+    u.w = L.sgu;
+    u.rows = 2 * sff;
+    u.cols = W;
+    u.x = st->x;
+    u.ldx = W;
+    u.y = st->sact;
+    u.ldy = sff;
+    u.T = T;
+    u.terms = terms_for(st, T);
+    u.glu = 1;
+    u.glu_limit = sp.shared_limit;
+    u.glu_alpha = sp.act_alpha;
+    TL_TRY(tl_launch_dense_gemm(u, s));
     TL_TRY(project(st, L.sdown, W, sff, st->sact, sff, st->sout, W, T, s));
     n.a = st->sout;
   }

@@ -15,7 +15,7 @@
 namespace {
 
 constexpr int SWA_WAVES = 4;
-constexpr int SWA_MAX_VR = 4;  // value columns per lane: vdim <= 256
+constexpr int SWA_MAX_VR = 8;  // value columns per lane: vdim <= 512
 
 __device__ __forceinline__ void swa_st_agent(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
