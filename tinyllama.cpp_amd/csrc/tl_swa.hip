@@ -41,9 +41,20 @@ __device__ __forceinline__ void swa_merge_records(const SwaArgs& a, int t, int h
   for (int d0 = 0; d0 < a.vdim; d0 += 64) {  // every lane stays in the loop: a shuffle reads nothing from a lane that has left
     const int d = d0 + lane;
     float acc = 0.0f;
-    for (int z = 0; z < a.nsplit; ++z) {
-      const float f = __shfl(fz, z);
-      if (d < a.vdim) acc += swa_ld_agent(rec + (size_t)z * rs + 2 + d) * f;
+    for (int z0 = 0; z0 < a.nsplit; z0 += 8) {  // eight records' values in flight together (clamped index, weight 0 beyond)
+      float v[8], f[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int z = z0 + u < a.nsplit ? z0 + u : a.nsplit - 1;
+        v[u] = d < a.vdim ? swa_ld_agent(rec + (size_t)z * rs + 2 + d) : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float fu = __shfl(fz, z0 + u < a.nsplit ? z0 + u : 0);
+        f[u] = z0 + u < a.nsplit ? fu : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc += v[u] * f[u];  // in split order
     }
     if (d < a.vdim) op[d] = acc / L;
   }
