@@ -1975,14 +1975,18 @@ extern "C" int tl_model_prefill_rows(tl_model* m, const int* tokens_host, int nu
   const int C = tl_stack_chunk(m->stack);
   const size_t V = (size_t)m->cfg.vocab_size;
   TL_TRY(upload_tokens(m, tokens_host, num_tokens, m->stream));
-  if (n_rows > 0 && m->pf.rows_cap < C) {
+  // the row list and logits of one chunk: as many rows as the largest request so far wanted from a chunk (at most C)
+  const int need = n_rows < C ? n_rows : C;
+  if (need > m->pf.rows_cap) {
+    TL_HIP(hipStreamSynchronize(m->stream));
     hipFree(m->pf.rows);
     hipFree(m->pf.logits_all);
     m->pf.rows = nullptr;
     m->pf.logits_all = nullptr;
-    TL_HIP(hipMalloc(&m->pf.rows, sizeof(int) * (size_t)C));
-    TL_HIP(hipMalloc(&m->pf.logits_all, sizeof(float) * (size_t)C * V));
-    m->pf.rows_cap = C;
+    m->pf.rows_cap = 0;
+    TL_HIP(hipMalloc(&m->pf.rows, sizeof(int) * (size_t)need));
+    TL_HIP(hipMalloc(&m->pf.logits_all, sizeof(float) * (size_t)need * V));
+    m->pf.rows_cap = need;
   }
   int r0 = 0;
   for (int t0 = 0; t0 < num_tokens; t0 += C) {

@@ -48,7 +48,10 @@ struct TlStack {
   std::vector<void*> allocs;
   bool finalized = false;
   int terms = 1;
-  int chunk = 512;
+  // tokens of a prompt that go through the layers together. Measured at width 4096 with 16 experts (top 4): 105.9 k tokens/s
+  // at 512, 140.4 k at 1024, 171.6 k at 2048 -- the experts' grouped GEMMs see 4 x the tokens per expert, the dense ones
+  // enough tiles for the 128 x 128 shape.
+  int chunk = 2048;
   bool gemv_decode = true;
   // workspaces for one chunk
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
