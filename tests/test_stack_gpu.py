@@ -243,7 +243,7 @@ def test_prompt_against_token_by_token_decoding(env, variant, gemv):
     """Every position decoded alone through the captured step (replayed once per token, prefill work in between) equals the
     prompt pass; positions run far beyond every window of the configuration."""
     cfg = small_config(env["synth"], variant)
-    m, _, orc = make(env, cfg, seed=13, TL_STACK_GEMV=gemv)
+    m, _, orc = make(env, cfg, seed=13, TL_STACK_GEMV=gemv, TL_STACK_FUSE_ROUTER=gemv)  # 0: also the router as its own launch
     assert m.graph_captured()
     rng = np.random.default_rng(2)
     n = 330 if variant == "wide" else 90

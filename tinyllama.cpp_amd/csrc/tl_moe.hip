@@ -13,6 +13,7 @@
 #include <math.h>
 
 #include "tl_bf16.h"
+#include "tl_route.h"
 #include "tl_stack.h"
 
 namespace {
@@ -38,53 +39,7 @@ __global__ __launch_bounds__(1024) void router_kernel(const RouterArgs a, int ve
     if (lane == 0) z[e] = s + (a.b ? a.b[e] : 0.0f);
   }
   __syncthreads();
-  if (wave == 0) {
-    // `top` rounds: the lanes scan the experts not yet chosen for the largest logit (lower index wins among equals)
-    float mx = 0.0f, denom = 0.0f, mine = 0.0f;
-    int my_id = -1;
-    for (int j = 0; j < a.top; ++j) {
-      float bv = -INFINITY;
-      int bi = 0x7fffffff;
-      for (int e = lane; e < a.experts; e += 64) {
-        const float v = z[e];
-        if (v > bv || (v == bv && e < bi)) {
-          bv = v;
-          bi = e;
-        }
-      }
-#pragma unroll
-      for (int o = 32; o >= 1; o >>= 1) {
-        const float ov = __shfl_xor(bv, o);
-        const int oi = __shfl_xor(bi, o);
-        if (ov > bv || (ov == bv && oi < bi)) {
-          bv = ov;
-          bi = oi;
-        }
-      }
-      if (bi == 0x7fffffff) bi = 0;  // only when every logit is NaN
-      if (j == 0) mx = bv;
-      const float p = expf(bv - mx);
-      denom += p;
-      if (lane == j % 64 && j < 64) {
-        mine = p;
-        my_id = bi;
-      }
-      if (j >= 64 && lane == 0) {  // more than 64 choices: written unnormalised, fixed up below
-        a.ids[t * a.top + j] = bi;
-        a.wts[t * a.top + j] = p;
-      }
-      if (lane == 0) z[bi] = -INFINITY;  // chosen: out of the next rounds
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
-    if (lane < a.top && lane < 64) {
-      a.ids[t * a.top + lane] = my_id;
-      a.wts[t * a.top + lane] = mine / denom;
-    }
-    if (a.top > 64 && lane == 0)
-      for (int j = 64; j < a.top; ++j) a.wts[t * a.top + j] /= denom;
-  }
+  if (wave == 0) tl_route_select(z, a.experts, a.top, a.ids + (size_t)t * a.top, a.wts + (size_t)t * a.top, lane);
 }
 
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ ids, int n_slots, int experts,

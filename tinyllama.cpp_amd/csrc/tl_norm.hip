@@ -4,6 +4,8 @@
 // whose launches are nothing but a chain of memory round trips); a row is staged in LDS, so that it is read from memory once.
 #include <math.h>
 
+#include "tl_bf16.h"
+#include "tl_route.h"
 #include "tl_stack.h"
 
 namespace {
@@ -26,7 +28,7 @@ inline int row_threads(int rows) { return rows <= 8 ? 1024 : 256; }
 __global__ __launch_bounds__(1024) void embed_norm_kernel(const unsigned short* __restrict__ table, int vocab, int width,
                                                          const int* __restrict__ tokens, const float* __restrict__ w,
                                                          float eps, float* __restrict__ x) {
-  extern __shared__ float row[];
+  extern __shared__ __attribute__((aligned(16))) float row[];
   __shared__ float red[kMaxWaves];
   const int t = blockIdx.x, tok = tokens[t];
   const bool in = tok >= 0 && tok < vocab;
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(1024) void qkv_post_kernel(const QkvPostArgs a) {
 }
 
 __global__ __launch_bounds__(1024) void resid_norm_kernel(const ResidNormArgs a) {
-  extern __shared__ float row[];
+  extern __shared__ __attribute__((aligned(16))) float row[];
   __shared__ float red[kMaxWaves];
   const int t = blockIdx.x;
   float ss = 0.0f;
@@ -97,12 +99,30 @@ __global__ __launch_bounds__(1024) void resid_norm_kernel(const ResidNormArgs a)
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)a.width + a.eps);
   float* x = a.x + (size_t)t * a.width;
-  for (int c = threadIdx.x; c < a.width; c += blockDim.x) x[c] += row[c] * inv * (1.0f + a.w[c]);
+  for (int c = threadIdx.x; c < a.width; c += blockDim.x) {
+    const float xn = x[c] + row[c] * inv * (1.0f + a.w[c]);
+    x[c] = xn;
+    row[c] = xn;  // the updated row stays in LDS for the router below
+  }
+  if (!a.route.w) return;
+  // ---- the router of the feed-forward that follows: logits = W_r x + b over the row in LDS, a wave per expert in turn ----
+  __syncthreads();
+  float* z = row + ((a.width + 3) & ~3);  // [experts]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const bool vec = (a.width & 7) == 0 && ((size_t)a.route.w & 15) == 0;
+  for (int e = wave; e < a.route.experts; e += nwaves) {
+    float sdot;
+    tl_wave_dot_rows<1>(a.route.w + (size_t)e * a.width, 0, 1, row, a.width, vec, lane, &sdot);
+    if (lane == 0) z[e] = sdot + (a.route.b ? a.route.b[e] : 0.0f);
+  }
+  __syncthreads();
+  if (wave == 0)
+    tl_route_select(z, a.route.experts, a.route.top, a.route.ids + (size_t)t * a.route.top, a.route.wts + (size_t)t * a.route.top, lane);
 }
 
 __global__ __launch_bounds__(1024) void norm_rows_kernel(const float* __restrict__ x, int width, const int* __restrict__ rows,
                                                         const float* __restrict__ w, float eps, float* __restrict__ out) {
-  extern __shared__ float row[];
+  extern __shared__ __attribute__((aligned(16))) float row[];
   __shared__ float red[kMaxWaves];
   const int i = blockIdx.x;
   const float* xr = x + (size_t)(rows ? rows[i] : i) * width;
@@ -144,7 +164,14 @@ int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s) {
   TL_REQUIRE(a.x && a.w && a.T > 0 && (a.a || a.slots), "resid_norm: bad arguments");
   TL_REQUIRE(a.width > 0 && a.width <= kMaxRowFloats, "resid_norm: width %d outside (0, %d]", a.width, kMaxRowFloats);
   TL_REQUIRE(!a.slots || (a.slot_w && a.top > 0), "resid_norm: expert slots without weights");
-  resid_norm_kernel<<<a.T, row_threads(a.T), sizeof(float) * a.width, s>>>(a);
+  size_t lds = sizeof(float) * a.width;
+  if (a.route.w) {
+    TL_REQUIRE(a.route.ids && a.route.wts && a.route.experts > 0 && a.route.top > 0 && a.route.top <= a.route.experts,
+               "resid_norm: bad router arguments");
+    lds = sizeof(float) * (((a.width + 3) & ~3) + a.route.experts);
+    TL_REQUIRE(lds <= 64 * 1024, "resid_norm: width %d + %d experts do not fit the staged row", a.width, a.route.experts);
+  }
+  resid_norm_kernel<<<a.T, row_threads(a.T), lds, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }

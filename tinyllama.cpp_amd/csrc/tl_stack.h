@@ -79,6 +79,15 @@ struct QkvPostArgs {
   const float* lambda;   // device scalar (vmix == 2)
 };
 int tl_launch_qkv_post(const QkvPostArgs& a, hipStream_t s);
+// (declared here because the residual norm may carry it; the launcher is tl_moe.hip's)
+struct RouterArgs {
+  const float* x;        // [T][width]
+  int T, width, experts, top;
+  const uint16_t* w;     // bf16 [experts][width]
+  const float* b;        // [experts]
+  int* ids;              // [T][top] chosen experts, largest logit first
+  float* wts;            // [T][top] softmax over the chosen logits
+};
 struct ResidNormArgs {
   float* x;              // [T][width] residual stream, updated in place: x += y / rms(y) * (1 + w)
   int T, width;
@@ -88,6 +97,9 @@ struct ResidNormArgs {
   int top;
   const float* w;
   float eps;
+  // optional: the router of the feed-forward that reads the updated x rides in this launch (the row is in LDS already):
+  // route.w != NULL -> route.ids / route.wts [T][top] as tl_launch_router writes them (route.x / T / width are ignored)
+  RouterArgs route;
 };
 int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s);
 // out[i] = x[rows[i]] / rms * (1 + w)   (rows == NULL: row i)
@@ -95,14 +107,6 @@ int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, c
                         hipStream_t s);
 
 // ---- tl_moe.hip --------------------------------------------------------------------------------------------------------
-struct RouterArgs {
-  const float* x;        // [T][width]
-  int T, width, experts, top;
-  const uint16_t* w;     // bf16 [experts][width]
-  const float* b;        // [experts]
-  int* ids;              // [T][top] chosen experts, largest logit first
-  float* wts;            // [T][top] softmax over the chosen logits
-};
 int tl_launch_router(const RouterArgs& a, hipStream_t s);
 // slots (t * top + j) grouped by expert: off[experts + 1], slot_of[T * top]
 int tl_launch_moe_plan(const int* ids, int n_slots, int experts, int* off, int* slot_of, hipStream_t s);

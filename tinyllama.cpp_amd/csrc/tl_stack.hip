@@ -53,6 +53,7 @@ struct TlStack {
   // enough tiles for the 128 x 128 shape.
   int chunk = 2048;
   bool gemv_decode = true;
+  bool fuse_router = true;  // TL_STACK_FUSE_ROUTER=0: the router as a launch of its own (A/B, tests)
   // workspaces for one chunk
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
   float *act_buf = nullptr, *eout = nullptr, *sact = nullptr, *sout = nullptr;
@@ -206,6 +207,7 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
     return fail(rc);
   if (const char* e = getenv("TL_STACK_CHUNK")) st->chunk = atoi(e) > 0 ? atoi(e) : st->chunk;
   if (const char* e = getenv("TL_STACK_GEMV")) st->gemv_decode = atoi(e) != 0;
+  if (const char* e = getenv("TL_STACK_FUSE_ROUTER")) st->fuse_router = atoi(e) != 0;
   *out = st;
   return 0;
 }
@@ -435,7 +437,7 @@ int moe_layer(TlStack* st, Layer& L, int T, hipStream_t s) {
   r.b = L.router_b;
   r.ids = st->ids;
   r.wts = st->wts;
-  TL_TRY(tl_launch_router(r, s));
+  if (!st->fuse_router) TL_TRY(tl_launch_router(r, s));  // (otherwise it rode in the x += N1 launch)
   ResidNormArgs n = {};
   n.x = st->x;
   n.T = T;
@@ -583,6 +585,14 @@ int tl_stack_forward(TlStack* st, const int* tokens_dev, int T, int start_pos, c
     n.a = st->proj;
     n.w = L.norm1;
     n.eps = c.norm_eps;
+    if (sp.mlp == TL_MLP_MOE && st->fuse_router) {  // the router reads the row this launch has just finished
+      n.route.w = L.router;
+      n.route.b = L.router_b;
+      n.route.experts = sp.experts;
+      n.route.top = sp.top;
+      n.route.ids = st->ids;
+      n.route.wts = st->wts;
+    }
     TL_TRY(tl_launch_resid_norm(n, s));
     if (sp.mlp == TL_MLP_MOE) TL_TRY(moe_layer(st, L, T, s));
     if (st->hook) {
