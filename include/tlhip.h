@@ -243,29 +243,79 @@ int tl_model_batch_generate_greedy(tl_model* m, int n, const int* first_tokens_h
  *      (terms 1 = bf16 activations in the chunk GEMMs, 3 = FP32-grade), tl_model_device_ptr, tl_model_bytes_per_token and
  *      tl_model_free work as for a Llama model; the multi-sequence and tensor-parallel entry points refuse it. Weights are
  *      bf16 matrices [out][in] and stay bf16 in HBM; the residual stream, norms, router, scores and caches are FP32. ------ */
-enum tl_mixer_kind { TL_MIXER_SWA = 0 };            /* sliding-window attention, no rotation, key size != value size allowed */
-enum tl_mlp_kind { TL_MLP_NONE = 0, TL_MLP_MOE = 1 }; /* no feed-forward | routed experts (+ optional shared expert) */
+enum tl_mixer_kind {
+  TL_MIXER_SWA = 0,         /* windowed attention over a key/value cache (softmax or sigmoid weights, optional rotation) */
+  TL_MIXER_DELTA = 1        /* gated delta rule with a decay per key channel: a recurrent state per head, no cache of keys */
+};
+enum tl_mlp_kind { TL_MLP_NONE = 0, TL_MLP_MOE = 1, TL_MLP_DENSE = 2 }; /* none | routed experts (+ shared expert) | one gated unit */
+enum tl_block_kind {
+  TL_BLOCK_POST_NORM = 0,   /* x += N1(mixer(x)); x += N2(ff(x)): the sublayers read x, the norm is on their output */
+  TL_BLOCK_PARALLEL = 1     /* h = N1(x); x += mixer(h) + ff(h): one norm, both sublayers read its output */
+};
+enum tl_norm_kind {
+  TL_NORM_RMS_ONE_PLUS = 0, /* y / sqrt(mean(y^2) + eps) * (1 + w) */
+  TL_NORM_DYT = 1           /* tanh(alpha y) * w + b: elementwise, no mean or variance (tensors <name>, <name>.alpha, <name>.b) */
+};
+enum tl_attn_weight {
+  TL_ATTN_SOFTMAX = 0,      /* weights normalised over the visible keys */
+  TL_ATTN_SIGMOID = 1       /* weight of a visible key = sigmoid(score + bias[head]); not normalised */
+};
+enum tl_qk_norm {
+  TL_QK_NORM_NONE = 0,
+  TL_QK_NORM_WHOLE = 1,     /* RMS norm over the WHOLE q and the whole k projection, plain weights (mix.q.norm, mix.k.norm) */
+  TL_QK_NORM_HEAD_UNIT = 2  /* per head, after the rotation: x / sqrt(mean(x^2) + eps), no weights */
+};
+enum tl_route_kind {
+  TL_ROUTE_TOP_LOGITS = 0,  /* the `top` largest logits (+ bias); weights = softmax over the chosen logits */
+  TL_ROUTE_SOFTMAX_GROUPS = 1 /* scores = softmax over all experts; experts in `route_groups` equal groups of neighbours, a
+                               group's score its best expert's, only the best `route_keep` groups can be chosen from;
+                               weights = the chosen scores divided by their sum (+ 1e-20) */
+};
 typedef struct tl_layer_spec {
   int mixer;                /* tl_mixer_kind */
   int heads, kv_heads;      /* query heads, key/value heads (query head h reads head h / (heads / kv_heads)) */
   int dim, vdim;            /* per-head query/key size, value size */
   int window;               /* position i sees j with 0 <= i - j < window; <= 0: every j <= i */
   float scale;              /* score = (q . k) * scale */
-  int qk_norm;              /* 1: RMS norm over the WHOLE q and the whole k projection, plain weights */
+  int qk_norm;              /* tl_qk_norm */
   int v_mix;                /* 1: v <- (1 - lambda) v + lambda v_first, v_first = the first such layer's values of the token */
   int mlp;                  /* tl_mlp_kind */
-  int experts, top;         /* routed experts, experts per token (weights: softmax over the chosen logits) */
-  int expert_ff;            /* y = g * sigmoid(act_alpha * g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit) */
-  float expert_limit;
-  int shared_ff;            /* 0: no shared expert */
+  int experts, top;         /* routed experts, experts per token */
+  int expert_ff;            /* y = g * sigmoid(act_alpha * g) * (u + glu_up_add), g = min(gate, limit), u = clamp(up, -limit, limit) */
+  float expert_limit;       /* (a limit of +infinity clamps nothing) */
+  int shared_ff;            /* 0: no shared expert. TL_MLP_DENSE: the one gated unit's size, its tensors are mlp.{gate,up,down} */
   float shared_limit;
   float act_alpha;
+  /* ---- everything below is zero for the plain softmax window attention of a post-norm block ---- */
+  float glu_up_add;         /* added to the up projection inside the gated unit (0 or 1) */
+  int block;                /* tl_block_kind */
+  int weights_of;           /* 1 + index of an EARLIER layer whose tensors (mixer, feed-forward, norms) this layer uses, with a
+                               cache or state of its own; 0: its own tensors. The rest of the entry must equal that layer's. */
+  int keep_first;           /* TL_MIXER_SWA: keys j < keep_first stay visible beyond the window (at their true positions) */
+  int attn_weight;          /* tl_attn_weight; TL_ATTN_SIGMOID reads the per-head bias mix.pb */
+  int values_are_keys;      /* 1: no value projection: v = the key as projected (before rotation and norm); vdim == dim */
+  int rot_dims;             /* rotary positions on the first rot_dims dimensions of each q / k head, dimension 2i paired with
+                               2i + 1, angle = position * f_i, f_i = rot_base^(-2i / rot_dims); 0: no rotation */
+  float rot_base;
+  float rot_factor;         /* > 0: context extension by frequency blending: with d(t) = rot_dims ln(rot_original / (2 pi t)) /
+                               (2 ln rot_base), lo = max(floor(d(rot_fast)), 0), hi = min(ceil(d(rot_slow)), rot_dims - 1),
+                               r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1): f_i <- f_i / rot_factor r_i + f_i (1 - r_i),
+                               and cos, sin are multiplied by 0.1 ln(rot_factor) + 1 */
+  float rot_original, rot_fast, rot_slow;
+  int conv_taps;            /* TL_MIXER_DELTA: taps of the causal convolution over time on q, k, v (each followed by silu) */
+  int decay_rank, gate_rank; /* TL_MIXER_DELTA: inner sizes of the two-step decay (a1, a2) and output gate (g1, g2) projections */
+  int route;                /* tl_route_kind */
+  int route_groups, route_keep;
+  int shared_gate;          /* 1: the shared expert's output is multiplied by sigmoid(w_sg . h) (mlp.shared.sg) */
 } tl_layer_spec;
 typedef struct tl_stack_config {
   int width, vocab, n_layers;
-  int max_positions;        /* rows of every layer's key/value cache */
-  float norm_eps;           /* every norm: x / sqrt(mean(x^2) + eps); block norms and the embedding / final norm use (1 + w) */
+  int max_positions;        /* rows of every attention layer's key/value cache */
+  float norm_eps;           /* every RMS norm: x / sqrt(mean(x^2) + eps) */
   const tl_layer_spec* layers;
+  int norm;                 /* tl_norm_kind of the block norms and the final norm */
+  int embed_norm;           /* 1: the embedding row is normalised (tensor embed.norm) before the first layer */
+  float logit_softcap;      /* > 0: logits <- cap * tanh(logits / cap) */
 } tl_stack_config;
 /* the operators such a model is built from, callable on their own (all FP32 in and out, weights bf16 [rows][cols]):
  * Y[T][rows] = X[T][cols] W^T; terms 1 / 3 = MFMA GEMM with bf16-rounded / three-term-split activations, 0 = FP32 GEMV (T = 1) */
@@ -277,15 +327,49 @@ int tl_swa_attention(const float* q_dev, const float* k_cache_dev, const float* 
                      int start_pos, int heads, int kv_heads, int dim, int vdim, int window, float scale, void* stream);
 /* x[t] += y[t] / sqrt(mean(y[t]^2) + eps) * (1 + weight) */
 int tl_resid_rmsnorm(float* x_dev, const float* y_dev, const float* weight_dev, int num_tokens, int width, float eps, void* stream);
-/* router: logits = W x + bias (FP32); ids [T][top] = the largest logits first (equal: lower index), weights = softmax over them */
+/* router (TL_ROUTE_TOP_LOGITS): logits = W x + bias (FP32); ids [T][top] = the largest logits first (equal: lower index), weights = softmax over them */
 int tl_moe_route(const float* x_dev, int num_tokens, int width, const void* w_bf16_dev, const float* bias_dev, int experts,
                  int top, int* ids_dev, float* weights_dev, void* stream);
 /* out[r][i] = g * sigmoid(alpha * g) * (u + 1), g = min(in[r][i], limit), u = clamp(in[r][ff + i], -limit, limit) */
 int tl_glu_clamp(const float* gate_up_dev, int rows, int ff, float limit, float alpha, float* out_dev, void* stream);
+/* tl_swa_attention with every option of the mixer: keys j < keep_first stay visible beyond the window; sigmoid != 0: the weight
+ * of a visible key is sigmoid(score + head_bias_dev[head]) and is not normalised */
+int tl_window_attention(const float* q_dev, const float* k_cache_dev, const float* v_cache_dev, float* out_dev, int num_tokens,
+                        int start_pos, int heads, int kv_heads, int dim, int vdim, int window, int keep_first, float scale,
+                        int sigmoid, const float* head_bias_dev, void* stream);
+/* router (TL_ROUTE_SOFTMAX_GROUPS), no bias: ids [T][top] largest score first, weights = chosen scores / their sum */
+int tl_moe_route_groups(const float* x_dev, int num_tokens, int width, const void* w_bf16_dev, int experts, int top, int groups,
+                        int keep, int* ids_dev, float* weights_dev, void* stream);
+/* out[t] = tanh(alpha x[t]) * w + b (alpha: one device float) */
+int tl_dyt_norm(const float* x_dev, const float* alpha_dev, const float* weight_dev, const float* bias_dev, float* out_dev,
+                int num_tokens, int width, void* stream);
+/* rotary positions as tl_layer_spec describes them (rot_factor <= 0: plain frequencies), in place on x [T][heads * dim] at
+ * positions start_pos.., then (unit_norm != 0) every head divided by its root mean square (eps inside the root) */
+int tl_rotary_heads(float* x_dev, int num_tokens, int start_pos, int heads, int dim, int rot_dims, float rot_base,
+                    float rot_factor, float rot_original, float rot_fast, float rot_slow, int unit_norm, float eps, void* stream);
+/* what precedes the gated delta rule, per token: p [T][ld] holds the projections q (kv_heads * dim) | k (kv_heads * dim) |
+ * v (heads * vdim) | beta (heads), a [T][heads * dim] the decay's pre-activation. q, k, v pass a causal convolution over time
+ * (w bf16 [channels][taps], channels = q | k | v, the last tap is the current token's; the inputs of the taps - 1 tokens before
+ * this call come from history [taps - 1][channels], oldest first, which afterwards holds the last taps - 1 inputs) and silu;
+ * q and k become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q also times dim^-1/2 -> qkv [T][channels];
+ * beta [T][heads] = sigmoid; g [T][heads * dim] = exp(-exp(a_log[head]) * softplus(a + dt_bias)) */
+int tl_delta_prepare(const float* p_dev, int ld, const float* a_dev, int num_tokens, int heads, int kv_heads, int dim, int vdim,
+                     int taps, const void* conv_bf16_dev, float* history_dev, const float* a_log_dev, const float* dt_bias_dev,
+                     float* qkv_dev, float* beta_dev, float* g_dev, void* stream);
+/* gated delta rule, token by token: per head h (q / k head h / (heads / kv_heads)) with state S [dim][vdim]:
+ * S <- diag(g_t) S; u = beta_t (v_t - S^T k_t); S <- S + k_t u^T; o_t = S^T q_t. q, k [T][kv_heads * dim], v, o [T][heads * vdim],
+ * beta [T][heads], g [T][heads * dim]; state_dev [heads][vdim][dim] (column-major per head), updated in place */
+int tl_delta_rule(const float* q_dev, const float* k_dev, const float* v_dev, const float* beta_dev, const float* g_dev,
+                  float* state_dev, float* o_dev, int num_tokens, int heads, int kv_heads, int dim, int vdim, void* stream);
+/* o[t][h] <- o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t][h]) per head, in place; o, gate [T][heads * vdim], w [vdim] */
+int tl_gated_head_norm(float* o_dev, const float* gate_dev, const float* weight_dev, int num_tokens, int heads, int vdim,
+                       float eps, void* stream);
+
 int tl_model_create_stack(const tl_stack_config* cfg, tl_model** out);
-/* tensors by checkpoint name: embed, embed.norm, final.norm, head, l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,q.norm,k.norm,vmix},
- * l<i>.mlp.router, l<i>.mlp.router.b, l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down}. type: TL_BF16 (matrices and
- * vectors) or TL_F32 (vectors). */
+/* tensors by checkpoint name: embed, embed.norm, final.norm, head, l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,q.norm,k.norm,vmix,pb},
+ * l<i>.mix.{q,k,v}.conv, l<i>.mix.{b,a1,a2,g1,g2,A_log,dt_bias,norm}, l<i>.mlp.router, l<i>.mlp.router.b,
+ * l<i>.mlp.e<j>.{gate,up,down}, l<i>.mlp.shared.{gate,up,down,sg}, l<i>.mlp.{gate,up,down}; a Dynamic Tanh norm <n> also has
+ * <n>.alpha and <n>.b. type: TL_BF16 (matrices and vectors) or TL_F32 (vectors). */
 int tl_model_set_tensor_named(tl_model* m, const char* name, int type, const long long* shape, int ndim, const void* host_data);
 /* a prompt, or a portion of one, at positions start_pos..: logits of the token rows listed in rows_host (ascending; NULL: the
  * last token when n_rows == 1, all tokens when n_rows == num_tokens) -> logits_host[n_rows][vocab]. The cache keeps what

@@ -29,12 +29,18 @@ class LayerSpec(C.Structure):
     _fields_ = [("mixer", C.c_int), ("heads", C.c_int), ("kv_heads", C.c_int), ("dim", C.c_int), ("vdim", C.c_int),
                 ("window", C.c_int), ("scale", C.c_float), ("qk_norm", C.c_int), ("v_mix", C.c_int), ("mlp", C.c_int),
                 ("experts", C.c_int), ("top", C.c_int), ("expert_ff", C.c_int), ("expert_limit", C.c_float),
-                ("shared_ff", C.c_int), ("shared_limit", C.c_float), ("act_alpha", C.c_float)]
+                ("shared_ff", C.c_int), ("shared_limit", C.c_float), ("act_alpha", C.c_float),
+                ("glu_up_add", C.c_float), ("block", C.c_int), ("weights_of", C.c_int), ("keep_first", C.c_int),
+                ("attn_weight", C.c_int), ("values_are_keys", C.c_int), ("rot_dims", C.c_int), ("rot_base", C.c_float),
+                ("rot_factor", C.c_float), ("rot_original", C.c_float), ("rot_fast", C.c_float), ("rot_slow", C.c_float),
+                ("conv_taps", C.c_int), ("decay_rank", C.c_int), ("gate_rank", C.c_int), ("route", C.c_int),
+                ("route_groups", C.c_int), ("route_keep", C.c_int), ("shared_gate", C.c_int)]
 
 
 class StackConfig(C.Structure):
     _fields_ = [("width", C.c_int), ("vocab", C.c_int), ("n_layers", C.c_int), ("max_positions", C.c_int),
-                ("norm_eps", C.c_float), ("layers", C.POINTER(LayerSpec))]
+                ("norm_eps", C.c_float), ("layers", C.POINTER(LayerSpec)), ("norm", C.c_int), ("embed_norm", C.c_int),
+                ("logit_softcap", C.c_float)]
 
 
 BF16 = 30
@@ -120,6 +126,16 @@ SIGNATURES = {
     "tl_resid_rmsnorm": [_fp, _fp, _fp, C.c_int, C.c_int, C.c_float, _vp],
     "tl_moe_route": [_fp, C.c_int, C.c_int, _vp, _fp, C.c_int, C.c_int, _ip, _fp, _vp],
     "tl_glu_clamp": [_fp, C.c_int, C.c_int, C.c_float, C.c_float, _fp, _vp],
+    "tl_window_attention": [_fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                            C.c_float, C.c_int, _fp, _vp],
+    "tl_moe_route_groups": [_fp, C.c_int, C.c_int, _vp, C.c_int, C.c_int, C.c_int, C.c_int, _ip, _fp, _vp],
+    "tl_dyt_norm": [_fp, _fp, _fp, _fp, _fp, C.c_int, C.c_int, _vp],
+    "tl_rotary_heads": [_fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float,
+                        C.c_float, C.c_int, C.c_float, _vp],
+    "tl_delta_prepare": [_fp, C.c_int, _fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _fp, _fp, _fp, _fp,
+                         _fp, _fp, _vp],
+    "tl_delta_rule": [_fp, _fp, _fp, _fp, _fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp],
+    "tl_gated_head_norm": [_fp, _fp, _fp, C.c_int, C.c_int, C.c_int, C.c_float, _vp],
 }
 
 # include/tlhip_debug.h: measurement / diagnostic hooks (not part of the boundary)

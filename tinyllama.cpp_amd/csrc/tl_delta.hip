@@ -1,0 +1,255 @@
+// tl_delta.hip — the gated delta rule with a decay per key channel, as a mixer of a layer-list model: a recurrent state
+// S [dim][vdim] per head instead of a cache of keys. Per token and head (q / k head = head / (heads / kv_heads)):
+//
+//     S <- diag(g) S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q        (the read-out sees the token's own write)
+//
+// with q, k from a short causal convolution over time + silu, made unit vectors per head (q also times dim^-1/2),
+// beta = sigmoid(.), g = exp(-exp(A_log[head]) * softplus(a + dt_bias)) per head and key channel. Everything that enters the
+// recurrence is FP32, and so is the state.
+//
+//   delta_pre    one workgroup per token: convolution (its last taps - 1 inputs of earlier calls come from a history that is
+//                part of the sequence's state), silu, the unit norms, beta and the decay.
+//   delta_scan   the recurrence. The columns of S (one per value channel) never mix: o_c = s_c . q, u_c = beta (v_c - s_c . k),
+//                s_c <- g * s_c + k u_c. Sixteen lanes share a column (each holds dim / 16 of its key channels in registers),
+//                four columns a wave, sixteen a workgroup, heads * vdim / 16 workgroups; the tokens are walked in order with
+//                the next token's operands in flight. The three dot products a token needs -- (g s) . k, (g s) . q and k . q,
+//                since o = (g s) . q + u (k . q) -- are reduced together over the sixteen lanes with row-local lane swaps, so a
+//                token costs one reduction latency, not two. A decode step is the same kernel with one token.
+//   gated norm   o / rms(o) * w * sigmoid(gate) per head, in front of the output projection.
+#include <math.h>
+
+#include "tl_bf16.h"
+#include "tl_stack.h"
+
+namespace {
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+__global__ __launch_bounds__(256) void delta_pre_kernel(const DeltaPreArgs a) {
+  extern __shared__ float row[];  // [channels] silu(conv)
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int qd = a.kv_heads * a.dim, vd = a.heads * a.vdim, C = 2 * qd + vd, H = a.taps - 1;
+  for (int c = tid; c < C; c += 256) {
+    const unsigned short* w = a.conv + (size_t)c * a.taps;
+    float acc = 0.0f;
+    for (int j = 0; j < a.taps; ++j) {
+      const int tt = t - H + j;  // token of this tap, relative to the call
+      const float in = tt >= 0 ? a.p[(size_t)tt * a.ld + c] : a.hist[(size_t)(H + tt) * C + c];
+      acc += tl_bf2f(w[j]) * in;
+    }
+    row[c] = acc * sigmoidf_(acc);
+    if (a.T == 1 && H > 0) {  // one token: this thread is the only reader of its channel's history, so it may shift it now
+      for (int j = 0; j + 1 < H; ++j) a.hist[(size_t)j * C + c] = a.hist[(size_t)(j + 1) * C + c];
+      a.hist[(size_t)(H - 1) * C + c] = a.p[c];
+    }
+  }
+  __syncthreads();
+  float* out = a.qkv + (size_t)t * C;
+  // q heads, then k heads: a wave per head
+  for (int hh = wave; hh < 2 * a.kv_heads; hh += 4) {
+    const float* x = row + (size_t)hh * a.dim;
+    float ss = 0.0f;
+    for (int d = lane; d < a.dim; d += 64) ss += x[d] * x[d];
+    ss = tl_wave_sum(ss);
+    float inv = 1.0f / sqrtf(ss + 1e-6f);
+    if (hh < a.kv_heads) inv *= 1.0f / sqrtf((float)a.dim);
+    for (int d = lane; d < a.dim; d += 64) out[(size_t)hh * a.dim + d] = x[d] * inv;
+  }
+  for (int c = 2 * qd + tid; c < C; c += 256) out[c] = row[c];
+  for (int h = tid; h < a.heads; h += 256) a.beta[(size_t)t * a.heads + h] = sigmoidf_(a.p[(size_t)t * a.ld + C + h]);
+  const int gd = a.heads * a.dim;
+  for (int c = tid; c < gd; c += 256) {
+    const float rate = expf(a.a_log[c / a.dim]);
+    a.g[(size_t)t * gd + c] = expf(-rate * softplusf_(a.a[(size_t)t * gd + c] + a.dt_bias[c]));
+  }
+}
+
+// after a call of several tokens: the history becomes the last taps - 1 inputs (a call shorter than that keeps the tail of
+// the old history in front). A thread owns a channel and walks its rows in ascending order, so no row is read after it was
+// overwritten.
+__global__ __launch_bounds__(256) void conv_history_kernel(const DeltaPreArgs a) {
+  const int qd = a.kv_heads * a.dim, C = 2 * qd + a.heads * a.vdim, H = a.taps - 1;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  for (int i = 0; i < H; ++i) {
+    const int src = a.T - H + i;  // token whose input lands in row i
+    a.hist[(size_t)i * C + c] = src >= 0 ? a.p[(size_t)src * a.ld + c] : a.hist[(size_t)(i + a.T) * C + c];
+  }
+}
+
+// sum over the 16 lanes of a row, result in all of them: lane swaps inside quads, then mirrored halves (no LDS round trip)
+__device__ __forceinline__ float row16_sum(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xf, 0xf, false));  // row_mirror
+  return x;
+}
+
+// E key channels per lane: dim <= 16 E. grid (vdim / 16 rounded up, heads), 256 threads.
+template <int E>
+__global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) {
+  const int tid = threadIdx.x, sub = tid & 15;
+  const int col = blockIdx.x * 16 + (tid >> 4), h = blockIdx.y;
+  const int kvh = h / (a.heads / a.kv_heads);
+  const bool live = col < a.vdim;           // lanes of a column beyond vdim compute on zeros and store nothing
+  const int d0 = sub * E;
+  float* sp = a.state + ((size_t)h * a.vdim + (live ? col : 0)) * a.dim;
+  float s[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) s[e] = (live && d0 + e < a.dim) ? sp[d0 + e] : 0.0f;
+  const float* qp = a.q + (size_t)kvh * a.dim;
+  const float* kp = a.k + (size_t)kvh * a.dim;
+  const float* gp = a.g + (size_t)h * a.dim;
+  const int gd = a.heads * a.dim;
+  float kn[E], qn[E], gn[E], vn, bn;
+  auto load = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const bool in = d0 + e < a.dim;
+      kn[e] = in ? kp[(size_t)t * a.ldq + d0 + e] : 0.0f;
+      qn[e] = in ? qp[(size_t)t * a.ldq + d0 + e] : 0.0f;
+      gn[e] = in ? gp[(size_t)t * gd + d0 + e] : 0.0f;
+    }
+    vn = live ? a.v[(size_t)t * a.ldv + (size_t)h * a.vdim + col] : 0.0f;
+    bn = a.beta[(size_t)t * a.heads + h];
+  };
+  load(0);
+  for (int t = 0; t < a.T; ++t) {
+    float kc[E], qc[E], gc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      kc[e] = kn[e];
+      qc[e] = qn[e];
+      gc[e] = gn[e];
+    }
+    const float vc = vn, bc = bn;
+    if (t + 1 < a.T) load(t + 1);
+    float sk = 0.0f, sq = 0.0f, kq = 0.0f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      s[e] *= gc[e];
+      sk += s[e] * kc[e];
+      sq += s[e] * qc[e];
+      kq += kc[e] * qc[e];
+    }
+    sk = row16_sum(sk);
+    sq = row16_sum(sq);
+    kq = row16_sum(kq);
+    const float u = bc * (vc - sk);
+#pragma unroll
+    for (int e = 0; e < E; ++e) s[e] += kc[e] * u;
+    if (live && sub == 0) a.o[(size_t)t * a.heads * a.vdim + (size_t)h * a.vdim + col] = sq + u * kq;
+  }
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (d0 + e < a.dim) sp[d0 + e] = s[e];
+  }
+}
+
+// a wave per (token, head)
+__global__ __launch_bounds__(256) void gated_head_norm_kernel(float* __restrict__ o, const float* __restrict__ gate,
+                                                             const float* __restrict__ w, int n_heads_total, int vdim,
+                                                             float eps) {
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (i >= n_heads_total) return;
+  float* x = o + (size_t)i * vdim;
+  const float* g = gate + (size_t)i * vdim;
+  float ss = 0.0f;
+  for (int d = lane; d < vdim; d += 64) ss += x[d] * x[d];
+  ss = tl_wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  for (int d = lane; d < vdim; d += 64) x[d] = x[d] * inv * w[d] * sigmoidf_(g[d]);
+}
+
+}  // namespace
+
+int tl_launch_delta_pre(const DeltaPreArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.p && a.a && a.conv && a.a_log && a.dt_bias && a.qkv && a.beta && a.g && a.T > 0, "delta_pre: bad arguments");
+  TL_REQUIRE(a.heads > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0 && a.dim > 0 && a.vdim > 0,
+             "delta_pre: %d heads over %d query/key heads, sizes %d / %d", a.heads, a.kv_heads, a.dim, a.vdim);
+  TL_REQUIRE(a.taps >= 1 && (a.taps == 1 || a.hist), "delta_pre: %d taps", a.taps);
+  const int C = 2 * a.kv_heads * a.dim + a.heads * a.vdim;
+  TL_REQUIRE(a.ld >= C + a.heads, "delta_pre: row stride %d below %d", a.ld, C + a.heads);
+  TL_REQUIRE(sizeof(float) * C <= 64 * 1024, "delta_pre: %d channels do not fit the staged row", C);
+  delta_pre_kernel<<<a.T, 256, sizeof(float) * C, s>>>(a);
+  if (a.T > 1 && a.taps > 1) conv_history_kernel<<<(C + 255) / 256, 256, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.q && a.k && a.v && a.beta && a.g && a.state && a.o && a.T > 0, "delta_scan: bad arguments");
+  TL_REQUIRE(a.heads > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0 && a.dim > 0 && a.vdim > 0 && a.heads <= 65535,
+             "delta_scan: %d heads over %d query/key heads, sizes %d / %d", a.heads, a.kv_heads, a.dim, a.vdim);
+  TL_REQUIRE(a.dim <= 256, "delta_scan: key size %d above 256", a.dim);
+  const dim3 grid((a.vdim + 15) / 16, a.heads);
+  const int e = (a.dim + 15) / 16;
+  if (e <= 1) delta_scan_kernel<1><<<grid, 256, 0, s>>>(a);
+  else if (e <= 2) delta_scan_kernel<2><<<grid, 256, 0, s>>>(a);
+  else if (e <= 4) delta_scan_kernel<4><<<grid, 256, 0, s>>>(a);
+  else if (e <= 8) delta_scan_kernel<8><<<grid, 256, 0, s>>>(a);
+  else delta_scan_kernel<16><<<grid, 256, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_gated_head_norm(float* o, const float* gate, const float* w, int T, int heads, int vdim, float eps, hipStream_t s) {
+  TL_REQUIRE(o && gate && w && T > 0 && heads > 0 && vdim > 0, "gated_head_norm: bad arguments");
+  const long long n = (long long)T * heads;
+  TL_REQUIRE(n <= 0x7fffffffLL, "gated_head_norm: too many heads");
+  gated_head_norm_kernel<<<(unsigned)((n + 3) / 4), 256, 0, s>>>(o, gate, w, (int)n, vdim, eps);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int tl_delta_prepare(const float* p_dev, int ld, const float* a_dev, int num_tokens, int heads, int kv_heads, int dim,
+                                int vdim, int taps, const void* conv_bf16_dev, float* history_dev, const float* a_log_dev,
+                                const float* dt_bias_dev, float* qkv_dev, float* beta_dev, float* g_dev, void* stream) {
+  DeltaPreArgs a = {};
+  a.p = p_dev;
+  a.ld = ld;
+  a.a = a_dev;
+  a.T = num_tokens;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.dim = dim;
+  a.vdim = vdim;
+  a.taps = taps;
+  a.conv = static_cast<const uint16_t*>(conv_bf16_dev);
+  a.hist = history_dev;
+  a.a_log = a_log_dev;
+  a.dt_bias = dt_bias_dev;
+  a.qkv = qkv_dev;
+  a.beta = beta_dev;
+  a.g = g_dev;
+  return tl_launch_delta_pre(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_gated_head_norm(float* o_dev, const float* gate_dev, const float* weight_dev, int num_tokens, int heads, int vdim,
+                                  float eps, void* stream) {
+  return tl_launch_gated_head_norm(o_dev, gate_dev, weight_dev, num_tokens, heads, vdim, eps, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_delta_rule(const float* q_dev, const float* k_dev, const float* v_dev, const float* beta_dev, const float* g_dev,
+                             float* state_dev, float* o_dev, int num_tokens, int heads, int kv_heads, int dim, int vdim,
+                             void* stream) {
+  DeltaScanArgs a = {};
+  a.q = q_dev;
+  a.k = k_dev;
+  a.ldq = kv_heads * dim;
+  a.v = v_dev;
+  a.ldv = heads * vdim;
+  a.beta = beta_dev;
+  a.g = g_dev;
+  a.state = state_dev;
+  a.o = o_dev;
+  a.T = num_tokens;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.dim = dim;
+  a.vdim = vdim;
+  return tl_launch_delta_scan(a, static_cast<hipStream_t>(stream));
+}

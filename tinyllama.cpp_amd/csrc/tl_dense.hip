@@ -31,10 +31,10 @@ __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest e
 __device__ __forceinline__ float bf2f(unsigned short h) { return tl_bf2f(h); }
 
 // y = g * sigmoid(alpha * g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit)  (tl_moe.hip has the operator)
-__device__ __forceinline__ float dense_glu(float g, float u, float limit, float alpha) {
+__device__ __forceinline__ float dense_glu(float g, float u, float limit, float alpha, float up_add) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
-  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  return g / (1.0f + expf(-alpha * g)) * (u + up_add);
 }
 
 constexpr int BK = 32, LDK = 40;  // LDK: padded row of a tile in LDS (80 B, keeps 16 B / 8 B alignment)
@@ -179,8 +179,12 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
 #pragma unroll
           for (int e = 0; e < 2; ++e)
             if (f + 2 * e + 1 < a.rows)
-              yr[(f >> 1) + e] = dense_glu(acc[i][j][gq * 4 + 2 * e], acc[i][j][gq * 4 + 2 * e + 1], a.glu_limit, a.glu_alpha);
+              yr[(f >> 1) + e] = dense_glu(acc[i][j][gq * 4 + 2 * e], acc[i][j][gq * 4 + 2 * e + 1], a.glu_limit, a.glu_alpha, a.glu_up_add);
           continue;
+        }
+        if (a.softcap > 0.0f) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][gq * 4 + e] = a.softcap * tanhf(acc[i][j][gq * 4 + e] / a.softcap);
         }
         if (v4 && f + 4 <= a.rows) {
           *reinterpret_cast<float4*>(yr + f) =
@@ -198,7 +202,8 @@ __global__ __launch_bounds__(256) void dense_gemm_kernel(const DenseArgs a) {
 // RW rows per wave, 4 waves per workgroup: 2 x RW sixteen-byte weight loads in flight per lane (tl_bf16.h)
 template <int RW>
 __global__ __launch_bounds__(256) void dense_gemv_kernel(const unsigned short* __restrict__ W, int rows, int cols,
-                                                         const float* __restrict__ x, float* __restrict__ y, int vec) {
+                                                         const float* __restrict__ x, float* __restrict__ y, int vec,
+                                                         float softcap) {
   const int lane = threadIdx.x & 63;
   const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
   if (row0 >= rows) return;
@@ -207,7 +212,7 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const unsigned short* _
   if (lane == 0) {
 #pragma unroll
     for (int r = 0; r < RW; ++r)
-      if (row0 + r < rows) y[row0 + r] = out[r];
+      if (row0 + r < rows) y[row0 + r] = softcap > 0.0f ? softcap * tanhf(out[r] / softcap) : out[r];
   }
 }
 
@@ -243,14 +248,14 @@ int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s) {
   return 0;
 }
 
-int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s) {
+int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s, float softcap) {
   TL_REQUIRE(w && x && y && rows > 0 && cols > 0, "dense gemv: bad arguments");
   const int vec = (cols & 7) == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0;
   // rows per wave: as many as still leave every CU a few workgroups
   const int cus = tl_num_cus();
-  if (rows >= 16 * 4 * cus) dense_gemv_kernel<4><<<(rows + 15) / 16, 256, 0, s>>>(w, rows, cols, x, y, vec);
-  else if (rows >= 8 * 4 * cus) dense_gemv_kernel<2><<<(rows + 7) / 8, 256, 0, s>>>(w, rows, cols, x, y, vec);
-  else dense_gemv_kernel<1><<<(rows + 3) / 4, 256, 0, s>>>(w, rows, cols, x, y, vec);
+  if (rows >= 16 * 4 * cus) dense_gemv_kernel<4><<<(rows + 15) / 16, 256, 0, s>>>(w, rows, cols, x, y, vec, softcap);
+  else if (rows >= 8 * 4 * cus) dense_gemv_kernel<2><<<(rows + 7) / 8, 256, 0, s>>>(w, rows, cols, x, y, vec, softcap);
+  else dense_gemv_kernel<1><<<(rows + 3) / 4, 256, 0, s>>>(w, rows, cols, x, y, vec, softcap);
   TL_HIP(hipGetLastError());
   return 0;
 }

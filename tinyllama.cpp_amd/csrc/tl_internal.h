@@ -66,7 +66,8 @@ enum TlScratchSlot {
   TL_SCRATCH_SAMPLE_PROBS,
   TL_SCRATCH_SAMPLE_PARAMS,
   TL_SCRATCH_GEMM_PART0,  // + 0..7: K-split partial tiles, one workspace per stream (tl_gemm.hip)
-  TL_SCRATCH_GEMM_PART7 = TL_SCRATCH_GEMM_PART0 + 7
+  TL_SCRATCH_GEMM_PART7 = TL_SCRATCH_GEMM_PART0 + 7,
+  TL_SCRATCH_ROTARY  // frequency table of tl_rotary_heads
 };
 int tl_scratch(int slot, size_t bytes, void** out);
 // tl_ops.hip: looks up the device address of tl_attention_noalloc's static workspace (called by tl_init, device current)

@@ -1,6 +1,7 @@
-// tl_norm.hip — the row-wise FP32 steps between the matrix products of a layer-list model. Every norm here is
+// tl_norm.hip — the row-wise FP32 steps between the matrix products of a layer-list model. An RMS norm here is
 // y = x / sqrt(mean(x^2) + eps) * weight, eps inside the root; "one-plus" weights are stored around zero and applied as
-// (1 + w). One workgroup per token row (256 threads for the rows of a prompt chunk, 1024 for the few rows of a decode step,
+// (1 + w). Norm-first blocks with the Dynamic Tanh norm (tanh(alpha x) * w + b: elementwise, no statistics) need no staged
+// row: embedding gather, residual sum and row gather carry the norm of the block that follows in the same pass. One workgroup per token row (256 threads for the rows of a prompt chunk, 1024 for the few rows of a decode step,
 // whose launches are nothing but a chain of memory round trips); a row is staged in LDS, so that it is read from memory once.
 #include <math.h>
 
@@ -139,7 +140,75 @@ __global__ __launch_bounds__(1024) void norm_rows_kernel(const float* __restrict
 
 constexpr int kMaxRowFloats = 16 * 1024;  // 64 KB of LDS for the staged row
 
+__device__ __forceinline__ float dyt_of(float x, float alpha, float w, float b) { return tanhf(alpha * x) * w + b; }
+
+// grid (column blocks of 256, T)
+__global__ __launch_bounds__(256) void embed_rows_kernel(const unsigned short* __restrict__ table, int vocab, int width,
+                                                        const int* __restrict__ tokens, float* __restrict__ x,
+                                                        const DytParams next, float* __restrict__ h) {
+  const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int tok = tokens[t];
+  const float v = (tok >= 0 && tok < vocab) ? __uint_as_float((unsigned)table[(size_t)tok * width + c] << 16) : 0.0f;
+  x[(size_t)t * width + c] = v;
+  if (next.alpha) h[(size_t)t * width + c] = dyt_of(v, *next.alpha, next.w[c], next.b[c]);
+}
+
+__global__ __launch_bounds__(256) void resid_sum_kernel(const ResidSumArgs a) {
+  const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= a.width) return;
+  const size_t i = (size_t)t * a.width + c;
+  float y = a.a ? a.a[i] : 0.0f;
+  if (a.slots) {
+    float e = 0.0f;
+    for (int j = 0; j < a.top; ++j) e += a.slot_w[t * a.top + j] * a.slots[((size_t)t * a.top + j) * a.width + c];
+    y += e;
+  }
+  if (a.b) y += a.b_gate ? a.b_gate[t] * a.b[i] : a.b[i];
+  const float xn = a.x[i] + y;
+  a.x[i] = xn;
+  if (a.next.alpha) a.h[i] = dyt_of(xn, *a.next.alpha, a.next.w[c], a.next.b[c]);
+}
+
+__global__ __launch_bounds__(256) void dyt_rows_kernel(const float* __restrict__ x, int width, const int* __restrict__ rows,
+                                                      const DytParams p, float* __restrict__ out) {
+  const int i = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  out[(size_t)i * width + c] = dyt_of(x[(size_t)(rows ? rows[i] : i) * width + c], *p.alpha, p.w[c], p.b[c]);
+}
+
 }  // namespace
+
+int tl_launch_embed_rows(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, float* x, const DytParams& next,
+                         float* h, hipStream_t s) {
+  TL_REQUIRE(table && tokens_dev && x && T > 0 && T <= 65535 && vocab > 0 && width > 0, "embed_rows: bad arguments");
+  TL_REQUIRE(!next.alpha || (next.w && next.b && h), "embed_rows: a norm without its weights or output");
+  embed_rows_kernel<<<dim3((width + 255) / 256, T), 256, 0, s>>>(table, vocab, width, tokens_dev, x, next, h);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_resid_sum(const ResidSumArgs& a, hipStream_t s) {
+  TL_REQUIRE(a.x && a.T > 0 && a.T <= 65535 && a.width > 0 && (a.a || a.b || a.slots), "resid_sum: bad arguments");
+  TL_REQUIRE(!a.slots || (a.slot_w && a.top > 0), "resid_sum: expert slots without weights");
+  TL_REQUIRE(!a.next.alpha || (a.next.w && a.next.b && a.h), "resid_sum: a norm without its weights or output");
+  resid_sum_kernel<<<dim3((a.width + 255) / 256, a.T), 256, 0, s>>>(a);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+int tl_launch_dyt_rows(const float* x, int width, const int* rows_dev, int n, const DytParams& p, float* out, hipStream_t s) {
+  TL_REQUIRE(x && out && p.alpha && p.w && p.b && n > 0 && n <= 65535 && width > 0, "dyt_rows: bad arguments");
+  dyt_rows_kernel<<<dim3((width + 255) / 256, n), 256, 0, s>>>(x, width, rows_dev, p, out);
+  TL_HIP(hipGetLastError());
+  return 0;
+}
+
+extern "C" int tl_dyt_norm(const float* x_dev, const float* alpha_dev, const float* weight_dev, const float* bias_dev,
+                           float* out_dev, int num_tokens, int width, void* stream) {
+  DytParams p = {alpha_dev, weight_dev, bias_dev};
+  return tl_launch_dyt_rows(x_dev, width, nullptr, num_tokens, p, out_dev, static_cast<hipStream_t>(stream));
+}
 
 int tl_launch_embed_norm(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, const float* w, float eps,
                          float* x, hipStream_t s) {

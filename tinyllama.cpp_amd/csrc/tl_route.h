@@ -53,3 +53,95 @@ __device__ __forceinline__ void tl_route_select(float* z, int experts, int top, 
     if (top > 64 && lane == 0)
       for (int j = 64; j < top; ++j) wts[j] /= denom;
 }
+
+// One wave: scores = softmax(z) over all experts (left in z[]); the experts form `groups` equal groups of neighbours, a
+// group's score is its best expert's, and only experts of the best `keep` groups (lower index among equals) can be chosen;
+// ids[top] = the chosen experts, largest score first (lower index among equals); wts = their scores divided by their sum
+// (+ 1e-20). key[experts] and gs[groups] are LDS scratch.
+__device__ __forceinline__ void tl_route_select_groups(float* z, float* key, float* gs, int experts, int top, int groups, int keep,
+                                                       int* ids, float* wts, int lane) {
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  float mx = -INFINITY;
+  for (int e = lane; e < experts; e += 64) mx = fmaxf(mx, z[e]);
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  float sum = 0.0f;
+  for (int e = lane; e < experts; e += 64) {
+    const float p = expf(z[e] - mx);
+    z[e] = p;
+    sum += p;
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) sum += __shfl_xor(sum, o);
+  const int per = experts / groups;
+  for (int e = lane; e < experts; e += 64) {
+    z[e] = z[e] / sum;
+    key[e] = -1.0f;  // below every score: not choosable until its group is kept
+  }
+  wave_sync();
+  for (int g = lane; g < groups; g += 64) {
+    float b = -1.0f;
+    for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, z[e]);
+    gs[g] = b;
+  }
+  wave_sync();
+  for (int r = 0; r < keep; ++r) {  // the best group not yet kept
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int g = lane; g < groups; g += 64) {
+      const float v = gs[g];
+      if (v > bv || (v == bv && g < bi)) {
+        bv = v;
+        bi = g;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oi = __shfl_xor(bi, o);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi == 0x7fffffff) bi = 0;
+    for (int e = bi * per + lane; e < (bi + 1) * per; e += 64) key[e] = z[e];
+    if (lane == 0) gs[bi] = -INFINITY;
+    wave_sync();
+  }
+  float denom = 0.0f;
+  for (int j = 0; j < top; ++j) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < experts; e += 64) {
+      const float v = key[e];
+      if (v > bv || (v == bv && e < bi)) {
+        bv = v;
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oi = __shfl_xor(bi, o);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (bi == 0x7fffffff) bi = 0;
+    const float sc = z[bi];
+    denom += sc;
+    if (lane == 0) {
+      ids[j] = bi;
+      wts[j] = sc;
+      key[bi] = -INFINITY;
+    }
+    wave_sync();
+  }
+  for (int j = lane; j < top; j += 64) wts[j] = wts[j] / (denom + 1e-20f);
+}

@@ -31,10 +31,12 @@ struct DenseArgs {
   // stores the clamped gated unit of each pair instead of the pair: y[item][i] (ldy >= rows / 2), see tl_launch_glu_act
   int glu;
   float glu_limit, glu_alpha;
+  float glu_up_add;      // 1 in the formula above; a design may add something else (0: the plain gated unit)
+  float softcap;         // > 0 (not with glu): y <- softcap * tanh(y / softcap)
 };
 int tl_launch_dense_gemm(const DenseArgs& a, hipStream_t s);
 // y[rows] = W x for one token, FP32 throughout (weights widened exactly)
-int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s);
+int tl_launch_dense_gemv(const uint16_t* w, int rows, int cols, const float* x, float* y, hipStream_t s, float softcap = 0.0f);
 
 // ---- tl_swa.hip --------------------------------------------------------------------------------------------------------
 struct SwaArgs {
@@ -55,9 +57,15 @@ struct SwaArgs {
   // optional: T * heads zeroed counters (left at zero by every launch): the last workgroup of a (token, head) to arrive merges
   // the records itself and the second launch falls away
   unsigned* done_cnt;
+  // keys j < keep_first stay visible to every later position, beyond the window (at their true positions)
+  int keep_first;
+  // sigmoid != 0: the weight of a visible key is sigmoid(score + head_bias[head]) (head_bias may be NULL) and is not
+  // normalised over the keys; 0: softmax
+  int sigmoid;
+  const float* head_bias;
 };
 int tl_launch_swa(const SwaArgs& a, hipStream_t s);
-int tl_swa_splits(int T, int window, int max_pos);  // splits worth having for T tokens over a cache of max_pos rows
+int tl_swa_splits(int T, int window, int max_pos, int keep_first = 0);  // splits worth having for T tokens over a cache of max_pos rows
 size_t tl_swa_ws_floats(int T, int heads, int vdim, int nsplit);
 
 // ---- tl_norm.hip -------------------------------------------------------------------------------------------------------
@@ -87,6 +95,12 @@ struct RouterArgs {
   const float* b;        // [experts]
   int* ids;              // [T][top] chosen experts, largest logit first
   float* wts;            // [T][top] softmax over the chosen logits
+  // kind = TL_ROUTE_SOFTMAX_GROUPS: scores = softmax over all experts; `groups` equal groups of neighbours ranked by their
+  // best score, only the best `keep` can be chosen from; wts = the chosen scores divided by their sum (+ 1e-20)
+  int kind, groups, keep;
+  // optional: one more row of weights whose logit becomes a gate per token, gate_out[t] = sigmoid(gate_w . x[t])
+  const uint16_t* gate_w;
+  float* gate_out;
 };
 struct ResidNormArgs {
   float* x;              // [T][width] residual stream, updated in place: x += y / rms(y) * (1 + w)
@@ -102,6 +116,30 @@ struct ResidNormArgs {
   RouterArgs route;
 };
 int tl_launch_resid_norm(const ResidNormArgs& a, hipStream_t s);
+// ---- norm-first blocks: Dynamic Tanh (elementwise, no statistics) and the plain residual sum ------------------------------
+struct DytParams {
+  const float* alpha;    // device scalar (NULL: no norm asked for)
+  const float* w;        // [width]
+  const float* b;        // [width]
+};
+// x[t] = embed[token[t]] (an id outside the table embeds as zeros); h[t] = tanh(alpha x[t]) * w + b when next.alpha is set
+int tl_launch_embed_rows(const uint16_t* table, int vocab, int width, const int* tokens_dev, int T, float* x, const DytParams& next,
+                         float* h, hipStream_t s);
+struct ResidSumArgs {
+  float* x;              // [T][width] residual stream: x += a + b * b_gate + sum_j slot_w[j] slots[j]
+  int T, width;
+  const float* a;        // optional [T][width]
+  const float* b;        // optional [T][width]
+  const float* b_gate;   // optional [T]: one factor per token on b
+  const float* slots;    // optional [T * top][width] expert outputs, weighted by slot_w
+  const float* slot_w;   // [T * top]
+  int top;
+  DytParams next;        // optional: h = norm of the updated x for the block that follows (saves that block a launch)
+  float* h;
+};
+int tl_launch_resid_sum(const ResidSumArgs& a, hipStream_t s);
+// out[i] = tanh(alpha x[rows[i]]) * w + b   (rows == NULL: row i)
+int tl_launch_dyt_rows(const float* x, int width, const int* rows_dev, int n, const DytParams& p, float* out, hipStream_t s);
 // out[i] = x[rows[i]] / rms * (1 + w)   (rows == NULL: row i)
 int tl_launch_norm_rows(const float* x, int width, const int* rows_dev, int n, const float* w, float eps, float* out,
                         hipStream_t s);
@@ -131,8 +169,63 @@ struct MoeDecodeArgs {
   float alpha;
   float* act;            // scratch [top * ff + sff]
   float* y;              // [width]
+  float up_add;          // the gated unit's (u + up_add)
+  const float* sgate;    // optional device scalar: factor on the shared expert's output
 };
 int tl_launch_moe_decode(const MoeDecodeArgs& a, hipStream_t s);
+
+// ---- tl_rope.hip -------------------------------------------------------------------------------------------------------
+// f[i] (i < rot_dims / 2) and the factor on cos / sin of a layer's rotary positions (tl_layer_spec: rot_*), computed in double
+void tl_rotary_frequencies(int rot_dims, double base, double factor, double original, double fast, double slow, float* f,
+                           float* mscale);
+struct RotaryArgs {
+  float* qk;             // [T][ld]: q heads (heads * dim) | k heads (kv_heads * dim) of a token, updated in place
+  int ld, heads, kv_heads, dim;
+  int rot_dims;          // the first rot_dims dimensions of a head rotate: (2i, 2i + 1) by position * freq[i]
+  const float* freq;     // device [rot_dims / 2]
+  float mscale;          // on cos and sin
+  int unit_norm;         // 1: after the rotation a head is divided by its root mean square (eps inside the root)
+  float eps;
+  float* kc;             // optional cache [max_pos][kv_heads * dim]: row pos receives the finished keys
+  float* vc;             // optional cache [max_pos][kv_heads * dim]: row pos receives the keys AS PROJECTED (values = keys)
+  const float* v_src;    // optional: a projected value row of vd floats per token (v_src + t * ld) ...
+  float* v_dst;          // ... copied to row pos of this cache [max_pos][vd]
+  int vd;
+  int T, start_pos;
+  const int* pos_dev;
+};
+int tl_launch_rotary(const RotaryArgs& a, hipStream_t s);
+
+// ---- tl_delta.hip ------------------------------------------------------------------------------------------------------
+struct DeltaPreArgs {
+  const float* p;        // [T][ld] projections of a token: q (kv_heads * dim) | k (kv_heads * dim) | v (heads * vdim) | beta (heads)
+  int ld;
+  const float* a;        // [T][heads * dim] decay pre-activation (before the bias)
+  int T, heads, kv_heads, dim, vdim, taps;
+  const uint16_t* conv;  // bf16 [channels][taps], channels = q | k | v in that order; the last tap is the current token's
+  float* hist;           // [taps - 1][channels] inputs of the tokens before this call (oldest first); updated
+  const float* a_log;    // [heads]
+  const float* dt_bias;  // [heads * dim]
+  float* qkv;            // out [T][channels]: silu(conv), q and k unit vectors per head (eps 1e-6), q times dim^-1/2
+  float* beta;           // out [T][heads] = sigmoid
+  float* g;              // out [T][heads * dim] = exp(-exp(a_log) softplus(a + dt_bias))
+};
+int tl_launch_delta_pre(const DeltaPreArgs& a, hipStream_t s);
+struct DeltaScanArgs {
+  const float* q;        // token t, head j at q + t * ldq + j * dim (kv_heads heads)
+  const float* k;
+  int ldq;
+  const float* v;        // token t, head h at v + t * ldv + h * vdim
+  int ldv;
+  const float* beta;     // [T][heads]
+  const float* g;        // [T][heads * dim]
+  float* state;          // [heads][vdim][dim]: column c of head h's S, contiguous over the key channels; updated
+  float* o;              // [T][heads * vdim]
+  int T, heads, kv_heads, dim, vdim;
+};
+int tl_launch_delta_scan(const DeltaScanArgs& a, hipStream_t s);
+// o[t][h] <- o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t][h]) per head (w [vdim] shared by the heads); in place
+int tl_launch_gated_head_norm(float* o, const float* gate, const float* w, int T, int heads, int vdim, float eps, hipStream_t s);
 
 // ---- tl_stack.hip: the engine ------------------------------------------------------------------------------------------
 struct TlStack;

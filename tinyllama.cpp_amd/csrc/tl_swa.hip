@@ -1,6 +1,10 @@
-// tl_swa.hip — sliding-window attention over a flat FP32 cache, without rotation: scores are (q . k) * scale, position i sees
-// the keys j with 0 <= i - j < window, ordinary softmax, everything in FP32. Key size (dim) and value size (vdim) are
-// independent; query head h reads key/value head h / (heads / kv_heads).
+// tl_swa.hip — sliding-window attention over a flat FP32 cache (rotation, if any, was applied before the keys were cached):
+// scores are (q . k) * scale, position i sees the keys j with 0 <= i - j < window and, when keep_first > 0, the keys
+// j < keep_first as well (the first tokens of the sequence stay visible at their true positions); the weights are an ordinary
+// softmax or, in sigmoid mode, sigmoid(score + bias[head]) without normalisation over the keys. Everything in FP32. Key size
+// (dim) and value size (vdim) are independent; query head h reads key/value head h / (heads / kv_heads).
+// Sigmoid mode runs through the softmax machinery with the running maximum pinned to 0: every correction factor is exp(0) = 1,
+// the partial sums of waves and splits are simply added, and the final division falls away.
 //
 // One workgroup of 4 waves per (token, head), for the tokens of a prompt chunk and for the single token of a decode step
 // alike. The visible keys are cut into pieces of 64; piece c belongs to wave c % 4. Within a piece a lane owns one key
@@ -56,7 +60,7 @@ __device__ __forceinline__ void swa_merge_records(const SwaArgs& a, int t, int h
 #pragma unroll
       for (int u = 0; u < 8; ++u) acc += v[u] * f[u];  // in split order
     }
-    if (d < a.vdim) op[d] = acc / L;
+    if (d < a.vdim) op[d] = a.sigmoid ? acc : acc / L;
   }
 }
 
@@ -71,6 +75,10 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   const int g = h / (a.heads / a.kv_heads);
   const int jlo = (a.window > 0 && i - a.window + 1 > 0) ? i - a.window + 1 : 0;
   const int n = i - jlo + 1;
+  // kept first keys that lie before the window: pieces [0, pf) walk them, pieces [pf, pieces) the window
+  const int nf = a.keep_first > 0 ? (a.keep_first < jlo ? a.keep_first : jlo) : 0;
+  const int pf = (nf + 63) >> 6;
+  const float hb = a.sigmoid && a.head_bias ? a.head_bias[h] : 0.0f;
   const int kld = a.kv_heads * a.dim, vld = a.kv_heads * a.vdim;
   const float* qp = a.q + (size_t)t * a.ldq + (size_t)h * a.dim;
   for (int d = tid; d < a.dim; d += 256) qs[d] = qp[d];
@@ -80,16 +88,17 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   float o[SWA_MAX_VR];
 #pragma unroll
   for (int r = 0; r < SWA_MAX_VR; ++r) o[r] = 0.0f;
-  const int pieces = (n + 63) >> 6;
+  const int pieces = pf + ((n + 63) >> 6);
   // nsplit > 1 (few tokens, long windows): workgroup z of (token, head) takes pieces [z * per, (z + 1) * per) and leaves its
   // (max, sum, unnormalised output) in ws for swa_combine_kernel
   const int nsplit = a.nsplit > 1 ? a.nsplit : 1;
   const int per = (pieces + nsplit - 1) / nsplit;
   const int c_lo = blockIdx.z * per, c_hi = c_lo + per < pieces ? c_lo + per : pieces;
   for (int c = c_lo + wave; c < c_hi; c += SWA_WAVES) {
-    const int j0 = jlo + c * 64;
+    const int j0 = c < pf ? c * 64 : jlo + (c - pf) * 64;
+    const int jend = c < pf ? nf - 1 : i;  // last visible key of this piece's region
     const int j = j0 + lane;
-    const bool valid = j <= i;
+    const bool valid = j <= jend;
     float sc = -INFINITY;
     if (valid) {
       const float* kp = a.kc + (size_t)j * kld + (size_t)g * a.dim;
@@ -119,15 +128,15 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
     float cm = sc;
 #pragma unroll
     for (int w = 32; w >= 1; w >>= 1) cm = fmaxf(cm, __shfl_xor(cm, w));
-    const float mn = fmaxf(m, cm);  // finite: lane 0 of a piece is always a visible key
-    const float p = valid ? expf(sc - mn) : 0.0f;
+    const float mn = a.sigmoid ? 0.0f : fmaxf(m, cm);  // finite: lane 0 of a piece is always a visible key
+    const float p = !valid ? 0.0f : a.sigmoid ? 1.0f / (1.0f + expf(-(sc + hb))) : expf(sc - mn);
     const float corr = expf(m - mn);  // m = -inf at the first piece: 0
     float ps = p;
 #pragma unroll
     for (int w = 32; w >= 1; w >>= 1) ps += __shfl_xor(ps, w);
     l = l * corr + ps;
     m = mn;
-    const int cnt = (i - j0 + 1) < 64 ? (i - j0 + 1) : 64;
+    const int cnt = (jend - j0 + 1) < 64 ? (jend - j0 + 1) : 64;
 #pragma unroll
     for (int r = 0; r < SWA_MAX_VR; ++r) o[r] *= corr;
     const float* vp = a.vc + (size_t)j0 * vld + (size_t)g * a.vdim;
@@ -214,8 +223,8 @@ __global__ __launch_bounds__(256) void swa_kernel(const SwaArgs a) {
   for (int d = tid; d < a.vdim; d += 256) {
     float acc = 0.0f;
 #pragma unroll
-    for (int w = 0; w < SWA_WAVES; ++w) acc += ow[w * a.vdim + d] * f[w];
-    op[d] = acc / L;
+    for (int w = 0; w < SWA_WAVES; ++w) acc += f[w] == 0.0f ? 0.0f : ow[w * a.vdim + d] * f[w];
+    op[d] = a.sigmoid ? acc : acc / L;
   }
 }
 
@@ -265,13 +274,20 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   const int last_q = start + last_i;
   const int klo = a.window > 0 && start + q0 - a.window + 1 > 0 ? start + q0 - a.window + 1 : 0;
   const int t_lo = klo >> 5, t_hi = last_q >> 5;
+  // kept first keys: their tiles of 32 positions below the window's first tile are walked before the window's tiles
+  // (virtual tile vt < tf is tile vt, vt >= tf is tile t_lo + vt - tf)
+  const int tf = a.keep_first > 0 ? (((a.keep_first + 31) >> 5) < t_lo ? ((a.keep_first + 31) >> 5) : t_lo) : 0;
+  const int nvt = tf + t_hi - t_lo + 1;
+  auto tile_of = [&](int vt) { return vt < tf ? vt : t_lo + vt - tf; };
+  const float hb = a.sigmoid && a.head_bias ? a.head_bias[head] : 0.0f;
+  // a row that no query of the tile can see (it carries weight 0) is read from a row that one of them can
+  auto clamp_row = [&](int pr) { return pr > last_q ? last_q : (pr < klo && pr >= a.keep_first) ? klo : pr; };
   const bool kvec = (a.dim & 3) == 0 && ((size_t)a.kc & 15) == 0;
   const bool vvec = (a.vdim % DB) == 0 && (DB == 1 || (((size_t)a.vc & 15) == 0 && (DB != 3)));
   // piece i (d = 8 i + 4 h + 0..3) of the lane's key row of a tile; rows outside [klo, last_q] are seen by no query of the
   // tile (masked below): their loads stay inside that range, so that nothing is read that the tile could not read
   auto load_k4 = [&](int tile, int i) -> swa_f32x4 {
-    const int pr = tile * 32 + r;
-    const int krow = pr > last_q ? last_q : pr < klo ? klo : pr;
+    const int krow = clamp_row(tile * 32 + r);
     const float* kp = a.kc + (size_t)krow * kld + (size_t)g * a.dim + 4 * h + 8 * i;
     const int d = 8 * i + 4 * h;
     swa_f32x4 kv;
@@ -288,8 +304,7 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
   auto load_v = [&](int p0, int e0, float (*vv)[DB]) __attribute__((always_inline)) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      int vrow = p0 + swa_acc_row(e0 + e, h);
-      vrow = vrow > last_q ? last_q : vrow < klo ? klo : vrow;
+      const int vrow = clamp_row(p0 + swa_acc_row(e0 + e, h));
       const float* vp = a.vc + (size_t)vrow * vld + (size_t)g * a.vdim + DB * r;
       if (vvec && DB * r < a.vdim) {
         if (DB == 4) {
@@ -311,10 +326,10 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
     }
   };
   swa_f32x4 kreg[PRE ? SWA_KREG4 : 1];
-  if (PRE && t_lo + wave <= t_hi) {
+  if (PRE && wave < nvt) {
 #pragma unroll
     for (int i = 0; i < SWA_KREG4; ++i)
-      if (i < dk) kreg[i] = load_k4(t_lo + wave, i);
+      if (i < dk) kreg[i] = load_k4(tile_of(wave), i);
   }
   for (int i = tid; i < 32 * dp; i += 256) {
     const int row = i / dp, d = i - row * dp;
@@ -328,7 +343,8 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
     for (int e = 0; e < 16; ++e) o[b][e] = 0.0f;
   float mrun = -INFINITY, lrun = 0.0f;
   const float* qrow = sm_q + r * qs + 4 * h;
-  for (int tile = t_lo + wave; tile <= t_hi; tile += SWA_WAVES) {
+  for (int vt = wave; vt < nvt; vt += SWA_WAVES) {
+    const int tile = tile_of(vt);
     const int p0 = tile * 32;
     swa_f32x16 s;
 #pragma unroll
@@ -341,10 +357,10 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
 #pragma unroll
           for (int c = 0; c < 4; ++c) s = __builtin_amdgcn_mfma_f32_32x32x2f32(kreg[i][c], qv[c], s, 0, 0, 0);
         }
-      if (tile + SWA_WAVES <= t_hi) {
+      if (vt + SWA_WAVES < nvt) {
 #pragma unroll
         for (int i = 0; i < SWA_KREG4; ++i)
-          if (i < dk) kreg[i] = load_k4(tile + SWA_WAVES, i);
+          if (i < dk) kreg[i] = load_k4(tile_of(vt + SWA_WAVES), i);
       }
     } else {
       for (int i = 0; i < dk; ++i) {
@@ -360,18 +376,19 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const int p = p0 + swa_acc_row(e, h);
-      const bool seen = p <= qpos && (a.window <= 0 || qpos - p < a.window);
+      const bool seen = p <= qpos && (a.window <= 0 || qpos - p < a.window || p < a.keep_first);
       s[e] = seen ? s[e] * a.scale : -INFINITY;
       tmax = fmaxf(tmax, s[e]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-    const float mnew = fmaxf(mrun, tmax);  // may still be -inf: a tile can lie wholly outside one query's window
+    // sigmoid mode: the maximum is pinned to 0 once the query has seen a key, so that no factor ever differs from 1
+    const float mnew = a.sigmoid ? (tmax == -INFINITY ? mrun : 0.0f) : fmaxf(mrun, tmax);  // may still be -inf: a tile can lie wholly outside one query's window
     const float corr = mrun == -INFINITY ? 0.0f : expf(mrun - mnew);
     mrun = mnew;
     float psum = 0.0f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      s[e] = s[e] == -INFINITY ? 0.0f : expf(s[e] - mnew);
+      s[e] = s[e] == -INFINITY ? 0.0f : a.sigmoid ? 1.0f / (1.0f + expf(-(s[e] + hb))) : expf(s[e] - mnew);
       psum += s[e];
     }
     lrun = lrun * corr + psum;
@@ -413,7 +430,7 @@ __global__ __launch_bounds__(256, 2) void swa_mfma_kernel(const SwaArgs a) {  //
         const float m2 = sm_m[w * 32 + r];
         L += m2 == -INFINITY ? 0.0f : sm_l[w * 32 + r] * expf(m2 - M);
       }
-      sm_inv[r] = 1.0f / L;
+      sm_inv[r] = a.sigmoid ? 1.0f : 1.0f / L;
     }
   }
   __syncthreads();
@@ -480,6 +497,7 @@ int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
              64 * SWA_MAX_VR);
   TL_REQUIRE(a.pos_dev || a.start_pos >= 0, "swa: negative start position");
   TL_REQUIRE(a.heads <= 65535, "swa: too many heads");
+  TL_REQUIRE(a.keep_first >= 0, "swa: negative number of kept first keys");
   if (swa_mfma_wanted(a)) {
     switch ((a.vdim + 31) / 32) {
       case 1: return launch_swa_mfma<1>(a, s);
@@ -500,9 +518,10 @@ int tl_launch_swa(const SwaArgs& a, hipStream_t s) {
   return 0;
 }
 
-int tl_swa_splits(int T, int window, int max_pos) {
+int tl_swa_splits(int T, int window, int max_pos, int keep_first) {
   if (T > 4) return 1;  // a chunk of a prompt has workgroups enough
-  const int keys = window > 0 && window < max_pos ? window : max_pos;
+  int keys = window > 0 && window < max_pos ? window : max_pos;
+  if (window > 0 && keep_first > 0) keys = keys + keep_first + 63 < max_pos ? keys + keep_first + 63 : max_pos;
   const int pieces = (keys + 63) / 64;
   int n = (pieces + SWA_WAVES - 1) / SWA_WAVES;  // a piece per wave and split
   return n < 1 ? 1 : n > 32 ? 32 : n;
@@ -528,6 +547,35 @@ extern "C" int tl_swa_attention(const float* q_dev, const float* k_cache_dev, co
   a.scale = scale;
   a.start_pos = start_pos;
   a.nsplit = tl_swa_splits(num_tokens, window, start_pos + num_tokens);
+  if (a.nsplit > 1) {
+    void* ws = nullptr;
+    TL_TRY(tl_scratch(TL_SCRATCH_ATTN, sizeof(float) * tl_swa_ws_floats(num_tokens, heads, vdim, a.nsplit), &ws));
+    a.ws = static_cast<float*>(ws);
+  }
+  return tl_launch_swa(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tl_window_attention(const float* q_dev, const float* k_cache_dev, const float* v_cache_dev, float* out_dev,
+                                   int num_tokens, int start_pos, int heads, int kv_heads, int dim, int vdim, int window,
+                                   int keep_first, float scale, int sigmoid, const float* head_bias_dev, void* stream) {
+  SwaArgs a = {};
+  a.q = q_dev;
+  a.ldq = heads * dim;
+  a.kc = k_cache_dev;
+  a.vc = v_cache_dev;
+  a.out = out_dev;
+  a.T = num_tokens;
+  a.heads = heads;
+  a.kv_heads = kv_heads;
+  a.dim = dim;
+  a.vdim = vdim;
+  a.window = window;
+  a.scale = scale;
+  a.start_pos = start_pos;
+  a.keep_first = keep_first;
+  a.sigmoid = sigmoid;
+  a.head_bias = head_bias_dev;
+  a.nsplit = tl_swa_splits(num_tokens, window, start_pos + num_tokens, keep_first);
   if (a.nsplit > 1) {
     void* ws = nullptr;
     TL_TRY(tl_scratch(TL_SCRATCH_ATTN, sizeof(float) * tl_swa_ws_floats(num_tokens, heads, vdim, a.nsplit), &ws));

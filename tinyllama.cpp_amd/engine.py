@@ -434,29 +434,74 @@ class Model:
             pass
 
 
-def stack_config_struct(config, max_pos):
+def _ralasun_spec(sp, i, L):
+    if L["type"] != "attention":
+        raise ValueError(f"layer {i}: unknown type {L['type']!r}")
+    mx, ml = L["mixer"], L.get("mlp")
+    sp.mixer, sp.heads, sp.kv_heads, sp.dim, sp.vdim = 0, mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+    sp.window = int((mx.get("mask") or {}).get("size", 0))
+    sp.scale, sp.qk_norm, sp.v_mix = float(mx["scale"]), 1, int(bool(mx.get("v_mix")))
+    sp.act_alpha, sp.glu_up_add = 1.702, 1.0
+    if ml is not None:
+        if ml.get("kind", "moe") != "moe":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {ml.get('kind')!r}")
+        sp.mlp, sp.experts, sp.top = 1, ml["router"]["experts"], ml["router"]["top"]
+        sp.expert_ff, sp.expert_limit = ml["expert"]["ff"], float(ml["expert"]["limit"])
+        sh = ml.get("shared")
+        if sh:
+            sp.shared_ff, sp.shared_limit = sh["ff"], float(sh["limit"])
+
+
+def _madalorn_spec(sp, i, L, tensors):
+    mx, ml = L["mixer"], L.get("mlp")
+    src = L.get("weights_of", i)
+    sp.weights_of = src + 1 if "weights_of" in L else 0
+    sp.block, sp.heads, sp.kv_heads, sp.dim, sp.vdim = 1, mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+    sp.act_alpha, sp.glu_up_add, sp.expert_limit, sp.shared_limit = 1.0, 0.0, float("inf"), float("inf")
+    if L["type"] == "attention":
+        sp.mixer, sp.scale, sp.attn_weight, sp.values_are_keys, sp.qk_norm = 0, float(mx["scale"]), 1, 1, 2
+        mask = mx.get("mask") or {}
+        sp.window, sp.keep_first = int(mask.get("size", 0)), int(mask.get("keep_first", 0))
+        rot = mx.get("rot")
+        if rot:
+            sp.rot_dims, sp.rot_base = rot["dims"], float(rot["base"])
+            sc = rot.get("scaling")
+            if sc:
+                sp.rot_factor, sp.rot_original = float(sc["factor"]), float(sc["original"])
+                sp.rot_fast, sp.rot_slow = float(sc["fast"]), float(sc["slow"])
+    elif L["type"] == "channel_delta":
+        sp.mixer, sp.conv_taps = 1, mx["conv"]
+        sp.decay_rank, sp.gate_rank = tensors[f"l{src}.mix.a1"].shape[0], tensors[f"l{src}.mix.g1"].shape[0]
+    else:
+        raise ValueError(f"layer {i}: unknown type {L['type']!r}")
+    if ml is not None:
+        if ml["kind"] == "dense":
+            sp.mlp, sp.shared_ff = 2, ml["ff"]
+        elif ml["kind"] == "moe":
+            r = ml["router"]
+            g = r.get("groups") or {"count": 1, "keep": 1}
+            sp.mlp, sp.route, sp.experts, sp.top, sp.route_groups, sp.route_keep = 1, 1, r["experts"], r["top"], g["count"], g["keep"]
+            sp.expert_ff = ml["expert"]["ff"]
+            if ml.get("shared"):
+                sp.shared_ff, sp.shared_gate = ml["shared"]["ff"], 1
+        else:
+            raise ValueError(f"layer {i}: unknown feed-forward kind {ml['kind']!r}")
+
+
+def stack_config_struct(config, max_pos, tensors=None):
     """The ctypes form (tl_stack_config) of a layer-list configuration given as config.json's dictionary; returns
     (struct, the array it points into). The C++ host does the same from the file (host/tl_stack_config.cpp); this one
-    serves tests and benches that build models in memory."""
+    serves tests and benches that build models in memory. `tensors` gives the inner sizes that only shapes name."""
     layers = config["layers"]
     arr = (capi.LayerSpec * len(layers))()
+    madalorn = config.get("architecture") == "Madalorn"
     for i, L in enumerate(layers):
-        if L["type"] != "attention":
-            raise ValueError(f"layer {i}: unknown type {L['type']!r}")
-        mx, ml, sp = L["mixer"], L.get("mlp"), arr[i]
-        sp.mixer, sp.heads, sp.kv_heads, sp.dim, sp.vdim = 0, mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
-        sp.window = int((mx.get("mask") or {}).get("size", 0))
-        sp.scale, sp.qk_norm, sp.v_mix = float(mx["scale"]), 1, int(bool(mx.get("v_mix")))
-        sp.act_alpha = 1.702
-        if ml is not None:
-            if ml.get("kind", "moe") != "moe":
-                raise ValueError(f"layer {i}: unknown feed-forward kind {ml.get('kind')!r}")
-            sp.mlp, sp.experts, sp.top = 1, ml["router"]["experts"], ml["router"]["top"]
-            sp.expert_ff, sp.expert_limit = ml["expert"]["ff"], float(ml["expert"]["limit"])
-            sh = ml.get("shared")
-            if sh:
-                sp.shared_ff, sp.shared_limit = sh["ff"], float(sh["limit"])
-    c = capi.StackConfig(config["width"], config["vocab"], len(layers), int(max_pos), float(config["norm"]["eps"]), arr)
+        if madalorn:
+            _madalorn_spec(arr[i], i, L, tensors or {})
+        else:
+            _ralasun_spec(arr[i], i, L)
+    c = capi.StackConfig(config["width"], config["vocab"], len(layers), int(max_pos), float(config["norm"]["eps"]), arr,
+                         1 if madalorn else 0, 0 if madalorn else 1, float(config.get("logit_softcap") or 0.0) if madalorn else 0.0)
     return c, arr
 
 
@@ -464,12 +509,12 @@ class StackModel(Model):
     """A layer-list model (tl_model_create_stack) behind the same handle and methods as Model. `config` is config.json's
     dictionary; tensors come by checkpoint name as uint16 arrays holding bf16 bits (or float32 arrays for vectors)."""
 
-    def __init__(self, config, max_pos=2048):
+    def __init__(self, config, max_pos=2048, tensors=None):
         _ensure_init()
         self.config = config
         self.cfg = {"vocab": config["vocab"], "hidden": config["width"], "n_layers": len(config["layers"]), "max_pos": max_pos}
         self.tp_rank, self.tp_size = 0, 1
-        c, self._keep = stack_config_struct(config, max_pos)
+        c, self._keep = stack_config_struct(config, max_pos, tensors)
         h = C.c_void_p()
         check(lib().tl_model_create_stack(C.byref(c), C.byref(h)), "tl_model_create_stack")
         self.h = h.value

@@ -16,6 +16,7 @@ const std::vector<ModelFamily>& model_families() {
   static const std::vector<ModelFamily> table = {
       {"llama", "gguf", load_llama_gguf},
       {"Ralasun", "folder", load_stack_folder},
+      {"Madalorn", "folder", load_stack_folder},
   };
   return table;
 }

@@ -1,11 +1,24 @@
-// tl_stack_config.cpp — loader of the layer-list family (tl_registry.hpp): config.json -> tl_stack_config, model.safetensors
-// -> tl_model_set_tensor_named. Every size and every constant that can differ between two models of the design is read from
-// the file; what the design fixes (the gate's 1.702, the whole-projection query/key norm) is set here.
+// tl_stack_config.cpp — loader of the layer-list families (tl_registry.hpp): config.json -> tl_stack_config, model.safetensors
+// -> tl_model_set_tensor_named. Every size and every constant that can differ between two models of a design is read from
+// the file (or, for an inner size the configuration does not name, from a tensor's shape); what a design fixes is set here.
 //
-// config.json: {"architecture", "width", "vocab", "norm": {"eps"}, "layers": [{"type": "attention",
-//   "mixer": {"heads", "kv_heads", "dim", "vdim", "scale", "mask": {"size"}, "v_mix"},
-//   "mlp": null | {"kind": "moe", "router": {"experts", "top"}, "expert": {"ff", "limit"}, "shared": null | {"ff", "limit"}}}]}
+// Ralasun   post-norm blocks with one-plus RMS norms, an embedding norm, softmax window attention with whole-projection q/k
+//           norm and value mixing, routed experts g * sigmoid(1.702 g) * (u + 1) with clamps, softmax over the chosen logits.
+//   {"architecture", "width", "vocab", "norm": {"eps"}, "layers": [{"type": "attention",
+//     "mixer": {"heads", "kv_heads", "dim", "vdim", "scale", "mask": {"size"}, "v_mix"},
+//     "mlp": null | {"kind": "moe", "router": {"experts", "top"}, "expert": {"ff", "limit"}, "shared": null | {"ff", "limit"}}}]}
+// Madalorn  parallel blocks behind one Dynamic Tanh norm; "attention" = sigmoid-weighted window attention whose values are
+//           the keys as projected, rotary positions with a context extension, per-head unit norm, kept first keys;
+//           "channel_delta" = gated delta rule with a decay per key channel; feed-forward dense or routed (softmax over all
+//           experts, groups) with a gated shared expert, plain silu gated units; layers may reuse an earlier layer's tensors;
+//           capped logits.
+//   {"architecture", "width", "vocab", "norm": {"eps"}, "logit_softcap", "layers": [{"type": "attention" | "channel_delta",
+//     "weights_of": j, "mixer": {"heads", "kv_heads", "dim", "vdim", "scale", "mask": {"size", "keep_first"},
+//     "rot": {"base", "dims", "scaling": {"factor", "original", "fast", "slow"}}, "conv"},
+//     "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "router": {"experts", "top", "groups": {"count", "keep"}},
+//     "expert": {"ff"}, "shared": null | {"ff"}}}]}
 #include <chrono>
+#include <cmath>
 #include <fstream>
 #include <sstream>
 #include <stdexcept>
@@ -18,7 +31,7 @@ namespace tlhost {
 
 namespace {
 
-constexpr float kGateAlpha = 1.702f;   // g * sigmoid(1.702 g): fixed by the design
+constexpr float kGateAlpha = 1.702f;   // Ralasun: g * sigmoid(1.702 g), fixed by the design
 constexpr int kDefaultContext = 4096;  // cache rows when the caller names no context length
 
 void hip_check(int rc, const std::string& what) {
@@ -26,39 +39,128 @@ void hip_check(int rc, const std::string& what) {
 }
 
 int geti(const Json& o, const char* key) { return (int)o.at(key).as_int(key); }
+float getf(const Json& o, const char* key) { return (float)o.at(key).as_double(key); }
+const Json* present(const Json& o, const char* key) {
+  const Json* v = o.find(key);
+  return (v && !v->is_null()) ? v : nullptr;
+}
 
-tl_layer_spec layer_from_json(const Json& L, int index) {
+tl_layer_spec ralasun_layer(const Json& L, int index, const SafeTensorsFile&) {
   const std::string where = "layers[" + std::to_string(index) + "]";
   tl_layer_spec sp = {};
   const std::string& type = L.at("type").as_string("type");
   if (type != "attention") throw std::runtime_error(where + ": unknown layer type \"" + type + "\"");
   const Json& mx = L.at("mixer");
   sp.mixer = TL_MIXER_SWA;
+  sp.block = TL_BLOCK_POST_NORM;
   sp.heads = geti(mx, "heads");
   sp.kv_heads = geti(mx, "kv_heads");
   sp.dim = geti(mx, "dim");
   sp.vdim = geti(mx, "vdim");
-  sp.scale = (float)mx.at("scale").as_double("scale");
-  const Json* mask = mx.find("mask");
-  sp.window = (mask && !mask->is_null()) ? geti(*mask, "size") : 0;
+  sp.scale = getf(mx, "scale");
+  const Json* mask = present(mx, "mask");
+  sp.window = mask ? geti(*mask, "size") : 0;
   const Json* vm = mx.find("v_mix");
   sp.v_mix = vm && vm->truthy();
-  sp.qk_norm = 1;
+  sp.qk_norm = TL_QK_NORM_WHOLE;
   sp.act_alpha = kGateAlpha;
-  const Json* ml = L.find("mlp");
-  if (ml && !ml->is_null()) {
+  sp.glu_up_add = 1.0f;
+  if (const Json* ml = present(L, "mlp")) {
     const Json* kind = ml->find("kind");
     if (kind && kind->as_string("kind") != "moe")
       throw std::runtime_error(where + ": unknown feed-forward kind \"" + kind->str + "\"");
     sp.mlp = TL_MLP_MOE;
+    sp.route = TL_ROUTE_TOP_LOGITS;
     sp.experts = geti(ml->at("router"), "experts");
     sp.top = geti(ml->at("router"), "top");
     sp.expert_ff = geti(ml->at("expert"), "ff");
-    sp.expert_limit = (float)ml->at("expert").at("limit").as_double("limit");
-    const Json* sh = ml->find("shared");
-    if (sh && !sh->is_null()) {
+    sp.expert_limit = getf(ml->at("expert"), "limit");
+    if (const Json* sh = present(*ml, "shared")) {
       sp.shared_ff = geti(*sh, "ff");
-      sp.shared_limit = (float)sh->at("limit").as_double("limit");
+      sp.shared_limit = getf(*sh, "limit");
+    }
+  }
+  return sp;
+}
+
+// an inner size that only a tensor's shape gives
+int tensor_rows(const SafeTensorsFile& file, const std::string& name) {
+  const SafeTensor* t = file.find(name);
+  if (!t || t->shape.size() != 2) throw std::runtime_error("model.safetensors: no matrix named " + name);
+  return (int)t->shape[0];
+}
+
+tl_layer_spec madalorn_layer(const Json& L, int index, const SafeTensorsFile& file) {
+  const std::string where = "layers[" + std::to_string(index) + "]";
+  tl_layer_spec sp = {};
+  const std::string& type = L.at("type").as_string("type");
+  const Json& mx = L.at("mixer");
+  int src = index;
+  if (const Json* wo = present(L, "weights_of")) {
+    src = (int)wo->as_int("weights_of");
+    if (src < 0 || src >= index) throw std::runtime_error(where + ": weights_of must name an earlier layer");
+    sp.weights_of = src + 1;
+  }
+  sp.block = TL_BLOCK_PARALLEL;
+  sp.heads = geti(mx, "heads");
+  sp.kv_heads = geti(mx, "kv_heads");
+  sp.dim = geti(mx, "dim");
+  sp.vdim = geti(mx, "vdim");
+  sp.act_alpha = 1.0f;  // silu
+  sp.glu_up_add = 0.0f;
+  sp.expert_limit = sp.shared_limit = INFINITY;
+  if (type == "attention") {
+    sp.mixer = TL_MIXER_SWA;
+    sp.scale = getf(mx, "scale");
+    sp.attn_weight = TL_ATTN_SIGMOID;
+    sp.values_are_keys = 1;
+    sp.qk_norm = TL_QK_NORM_HEAD_UNIT;
+    if (const Json* mask = present(mx, "mask")) {
+      sp.window = geti(*mask, "size");
+      if (const Json* kf = present(*mask, "keep_first")) sp.keep_first = (int)kf->as_int("keep_first");
+    }
+    if (const Json* rot = present(mx, "rot")) {
+      sp.rot_dims = geti(*rot, "dims");
+      sp.rot_base = getf(*rot, "base");
+      if (const Json* sc = present(*rot, "scaling")) {
+        sp.rot_factor = getf(*sc, "factor");
+        sp.rot_original = getf(*sc, "original");
+        sp.rot_fast = getf(*sc, "fast");
+        sp.rot_slow = getf(*sc, "slow");
+      }
+    }
+  } else if (type == "channel_delta") {
+    sp.mixer = TL_MIXER_DELTA;
+    sp.conv_taps = geti(mx, "conv");
+    const std::string p = "l" + std::to_string(src) + ".mix.";
+    sp.decay_rank = tensor_rows(file, p + "a1");
+    sp.gate_rank = tensor_rows(file, p + "g1");
+  } else {
+    throw std::runtime_error(where + ": unknown layer type \"" + type + "\"");
+  }
+  if (const Json* ml = present(L, "mlp")) {
+    const std::string& kind = ml->at("kind").as_string("kind");
+    if (kind == "dense") {
+      sp.mlp = TL_MLP_DENSE;
+      sp.shared_ff = geti(*ml, "ff");
+    } else if (kind == "moe") {
+      sp.mlp = TL_MLP_MOE;
+      sp.route = TL_ROUTE_SOFTMAX_GROUPS;
+      const Json& r = ml->at("router");
+      sp.experts = geti(r, "experts");
+      sp.top = geti(r, "top");
+      sp.route_groups = sp.route_keep = 1;
+      if (const Json* g = present(r, "groups")) {
+        sp.route_groups = geti(*g, "count");
+        sp.route_keep = geti(*g, "keep");
+      }
+      sp.expert_ff = geti(ml->at("expert"), "ff");
+      if (const Json* sh = present(*ml, "shared")) {
+        sp.shared_ff = geti(*sh, "ff");
+        sp.shared_gate = 1;
+      }
+    } else {
+      throw std::runtime_error(where + ": unknown feed-forward kind \"" + kind + "\"");
     }
   }
   return sp;
@@ -75,8 +177,13 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   const Json cfg = Json::parse(ss.str());
   const Json& layers = cfg.at("layers");
   if (layers.kind != Json::ARRAY || layers.arr.empty()) throw std::runtime_error("config.json: \"layers\" is empty");
+  const std::string arch = cfg.at("architecture").as_string("architecture");
+  const bool madalorn = arch == "Madalorn";
+  SafeTensorsFile file;
+  file.open(dir + "/model.safetensors");
   std::vector<tl_layer_spec> specs;
-  for (size_t i = 0; i < layers.arr.size(); ++i) specs.push_back(layer_from_json(layers.arr[i], (int)i));
+  for (size_t i = 0; i < layers.arr.size(); ++i)
+    specs.push_back(madalorn ? madalorn_layer(layers.arr[i], (int)i, file) : ralasun_layer(layers.arr[i], (int)i, file));
   tl_stack_config sc = {};
   sc.width = geti(cfg, "width");
   sc.vocab = geti(cfg, "vocab");
@@ -84,6 +191,10 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   sc.max_positions = max_context > 0 ? max_context : kDefaultContext;
   sc.norm_eps = (float)cfg.at("norm").at("eps").as_double("norm.eps");
   sc.layers = specs.data();
+  sc.norm = madalorn ? TL_NORM_DYT : TL_NORM_RMS_ONE_PLUS;
+  sc.embed_norm = madalorn ? 0 : 1;
+  if (madalorn)
+    if (const Json* cap = present(cfg, "logit_softcap")) sc.logit_softcap = (float)cap->as_double("logit_softcap");
 
   ModelConfig& mc = out->config;
   mc.architecture = cfg.at("architecture").as_string("architecture");
@@ -95,7 +206,7 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   mc.rms_norm_eps = sc.norm_eps;
   mc.num_attention_heads = specs[0].heads;
   mc.num_key_value_heads = specs[0].kv_heads;
-  mc.intermediate_size = specs[0].expert_ff;
+  mc.intermediate_size = specs[0].mlp == TL_MLP_DENSE ? specs[0].shared_ff : specs[0].expert_ff;
   mc.bos_token_id = -1;  // token ids in, token ids out: such a checkpoint carries no tokenizer
   mc.eos_token_id = -1;
   if (const Json* e = cfg.find("eos"))
@@ -104,8 +215,6 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   hip_check(tl_init(device), "tl_init");
   hip_check(tl_model_create_stack(&sc, &out->model), "tl_model_create_stack");
   try {
-    SafeTensorsFile file;
-    file.open(dir + "/model.safetensors");
     for (const SafeTensor& t : file.tensors()) {
       int type = -1;
       if (t.dtype == "BF16") type = TL_BF16;

@@ -334,6 +334,109 @@ def build_stack(config, seed=0, gain=1.0):
     return t
 
 
+def madalorn_attention(heads, kv_heads, dim, window=None, keep_first=0, rot_dims=None, base=10000.0, scaling=None, scale=None):
+    """The "mixer" entry of a Madalorn attention layer (values are the keys: vdim = dim). scaling: None or a dict
+    {factor, original, fast, slow}."""
+    mixer = {"dim": dim, "heads": heads, "kv_heads": kv_heads, "vdim": dim,
+             "scale": float(scale if scale is not None else dim ** -0.5),
+             "rot": {"base": float(base), "dims": int(dim if rot_dims is None else rot_dims)}}
+    if scaling:
+        mixer["rot"]["scaling"] = {k: (int(v) if k == "original" else float(v)) for k, v in scaling.items()}
+    if window is not None:
+        mixer["mask"] = {"size": int(window), "keep_first": int(keep_first)}
+    return mixer
+
+
+def madalorn_delta(heads, kv_heads, dim, vdim, conv=4):
+    return {"conv": int(conv), "dim": dim, "heads": heads, "kv_heads": kv_heads, "vdim": vdim}
+
+
+def madalorn_moe(experts, top, ff, shared_ff=0, groups=1, keep=1):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}},
+            "shared": {"ff": shared_ff} if shared_ff else None}
+
+
+def madalorn_layer(kind, mixer, mlp=None, weights_of=None):
+    L = {"type": kind, "mixer": mixer, "mlp": mlp}
+    if weights_of is not None:
+        L["weights_of"] = int(weights_of)
+    return L
+
+
+def madalorn_config(width, vocab, layers, eps=1e-6, softcap=30.0):
+    return {"architecture": "Madalorn", "layers": list(layers), "logit_softcap": float(softcap), "norm": {"eps": float(eps)},
+            "vocab": int(vocab), "width": int(width)}
+
+
+def build_madalorn(config, seed=0, gain=1.0, ranks=(8, 8)):
+    """Random tensors {checkpoint name: uint16 bf16 bits} of a Madalorn configuration. Layers with weights_of get none.
+    ranks: inner sizes of the decay and output-gate projections of delta layers."""
+    rng = np.random.default_rng(seed)
+    W, V = config["width"], config["vocab"]
+    t = {}
+
+    def mat(name, rows, cols, std=None):
+        t[name] = to_bf16(rng.standard_normal((rows, cols)).astype(np.float32) * (std or gain / np.sqrt(cols)))
+
+    def vec(name, n, centre, spread, shape=None):
+        a = to_bf16((centre + spread * rng.standard_normal(n)).astype(np.float32))
+        t[name] = a.reshape(shape) if shape is not None else a
+
+    def norm(name):
+        vec(name, W, 1.0, 0.1)
+        vec(name + ".b", W, 0.0, 0.05)
+        t[name + ".alpha"] = to_bf16(np.array(rng.uniform(0.4, 0.9), np.float32))
+
+    def glu(p, ff):
+        mat(p + "gate", ff, W, 2.0 / np.sqrt(W))
+        mat(p + "up", ff, W, 2.0 / np.sqrt(W))
+        mat(p + "down", W, ff)
+
+    mat("embed", V, W, 1.0)
+    norm("final.norm")
+    mat("head", V, W, 4.0 / np.sqrt(W))
+    for i, L in enumerate(config["layers"]):
+        if "weights_of" in L:
+            continue
+        mx, ml, p = L["mixer"], L.get("mlp"), f"l{i}."
+        H, G, d, dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+        norm(p + "norm1")
+        if L["type"] == "attention":
+            mat(p + "mix.q", H * d, W)
+            mat(p + "mix.k", G * d, W)
+            vec(p + "mix.pb", H, -1.0, 0.5)
+            mat(p + "mix.o", W, H * dv)
+        else:
+            ra, rg = ranks
+            mat(p + "mix.q", G * d, W)
+            mat(p + "mix.k", G * d, W)
+            mat(p + "mix.v", H * dv, W)
+            for n, c in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                mat(p + f"mix.{n}.conv", c, mx["conv"], 0.5)
+            mat(p + "mix.b", H, W)
+            vec(p + "mix.A_log", H, -0.5, 0.5)
+            vec(p + "mix.norm", dv, 1.0, 0.1)
+            mat(p + "mix.a1", ra, W)
+            mat(p + "mix.a2", H * d, ra)
+            vec(p + "mix.dt_bias", H * d, -1.0, 0.5)
+            mat(p + "mix.g1", rg, W)
+            mat(p + "mix.g2", H * dv, rg)
+            mat(p + "mix.o", W, H * dv)
+        if ml is None:
+            continue
+        if ml["kind"] == "dense":
+            glu(p + "mlp.", ml["ff"])
+        else:
+            E = ml["router"]["experts"]
+            for e in range(E):
+                glu(p + f"mlp.e{e}.", ml["expert"]["ff"])
+            mat(p + "mlp.router", E, W, 2.0 / np.sqrt(W))
+            if ml.get("shared"):
+                glu(p + "mlp.shared.", ml["shared"]["ff"])
+                mat(p + "mlp.shared.sg", 1, W)
+    return t
+
+
 def write_stack_dir(path, config, tensors):
     """config.json + model.safetensors (8-byte little-endian header length, JSON header, data) under `path`."""
     import json
