@@ -62,6 +62,8 @@ def rotary_frequencies(rot):
 
 def rotate(x, pos, rot):
     """x [T, heads, dim] at positions pos [T]; interleaved pairs (2i, 2i + 1) of the first rot.dims dimensions."""
+    if not rot:
+        return x.copy()
     f, m = rotary_frequencies(rot)
     n = rot["dims"]
     a = np.asarray(pos, np.float64)[:, None, None] * f[None, None, :]
@@ -162,8 +164,8 @@ class MadalornOracle:
         q = (h @ w[p + "q"].T).reshape(T, H, d)
         k = (h @ w[p + "k"].T).reshape(T, G, d)
         v = k.copy()
-        q = unit_rms(rotate(q, pos, mx["rot"]), self.eps)
-        k = unit_rms(rotate(k, pos, mx["rot"]), self.eps)
+        q = unit_rms(rotate(q, pos, mx.get("rot")), self.eps)
+        k = unit_rms(rotate(k, pos, mx.get("rot")), self.eps)
         self.k[i] = k if self.k[i] is None else np.concatenate([self.k[i], k])
         self.v[i] = v if self.v[i] is None else np.concatenate([self.v[i], v])
         mask = mx.get("mask") or {}
@@ -229,3 +231,13 @@ class MadalornOracle:
         z = self.norm("final.norm", x) @ self.w["head"].T
         cap = self.c.get("logit_softcap")
         return cap * np.tanh(z / cap) if cap else z
+
+    def generate_greedy(self, prompt, n_new):
+        """Arg-max continuation (first maximum), token by token after the prompt; resets the sequence first."""
+        self.reset()
+        logits = self.forward(list(prompt))[-1]
+        out = []
+        for _ in range(n_new):
+            out.append(int(np.argmax(logits)))
+            logits = self.forward([out[-1]])[0]
+        return out
