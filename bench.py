@@ -52,8 +52,10 @@ def parse():
     ap.add_argument("--prompt-len", type=int, default=4)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers in the CPU-baseline sample")
-    ap.add_argument("--family", default=None, choices=[None, "ralasun"],
-                    help="ralasun: prefill / decode throughput of the layer-list family at --sizes beside a Llama model of "
+    ap.add_argument("--family", default=None, choices=[None, "ralasun", "madalorn"],
+                    help="madalorn: prefill / decode throughput of that layer-list design at --sizes beside a Ralasun model of "
+                         "equal size (the closest existing model: same engine, bf16 weights, window attention, routed experts); "
+                         "ralasun: prefill / decode throughput of the layer-list family at --sizes beside a Llama model of "
                          "equal size (one GPU; prints its own JSON line; the default workload and line are untouched)")
     ap.add_argument("--sizes", default="s,m,l", help="with --family: comma-separated names out of s, m, l")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="with --family: prompt length of the prefill leg")
@@ -114,6 +116,119 @@ def _pool_bf16(S, n, std, rng, pool):
     return S.to_bf16(a * np.float32(std))
 
 
+def _time_stack_model(m, args, T, V, layers, per_tok, rng, exact_terms=3):
+    """Prefill (bf16 activations and FP32-grade) and greedy decode of a finalized layer-list model: a dict of rates."""
+    toks = rng.integers(0, V, T).astype(np.int32)
+    last_row = np.array([T - 1], np.int32)
+    r = {}
+    for terms, label in ((1, "bf16"), (exact_terms, "fp32_grade")):
+        m.set_prefill(terms, 1)
+        m.reset_kv()
+        m.prefill_rows(toks, 0, last_row)
+        best = 1e9
+        for _ in range(3):
+            m.reset_kv()
+            t0 = time.perf_counter()
+            m.prefill_rows(toks, 0, last_row)
+            best = min(best, time.perf_counter() - t0)
+        r[f"prefill_{label}_tokens_per_s"] = round(T / best, 1)
+        r[f"prefill_{label}_gemm_tflops"] = round(2.0 * T * per_tok * layers / best / 1e12, 2)
+    m.set_prefill(1, 1)
+    m.reset_kv()
+    first = int(np.argmax(m.prefill_rows(toks, 0, last_row)[0]))  # the cache now holds T positions
+    m.generate_greedy(first, T, args.warmup)
+    t0 = time.perf_counter()
+    m.generate_greedy(first, T + args.warmup, args.steps)
+    dt = time.perf_counter() - t0
+    wb, kb = m.bytes_per_token(T + args.warmup)
+    r.update(decode_tokens_per_s=round(args.steps / dt, 1), decode_us_per_token=round(dt / args.steps * 1e6, 1),
+             decode_bytes_per_token=int(wb + kb), decode_hbm_gbps=round((wb + kb) * args.steps / dt / 1e9, 1),
+             decode_frac_of_hbm_peak=round((wb + kb) * args.steps / dt / 1e9 / HBM_PEAK_GBPS, 4),
+             graph_nodes=m.graph_nodes())
+    return r, toks, first
+
+
+def _build_ralasun(S, engine, z, max_pos, rng, pool):
+    W, V = z["width"], z["vocab"]
+    layer = S.stack_layer(z["heads"], z["kv_heads"], z["dim"], z["vdim"], z["window"], v_mix=True, experts=z["experts"],
+                          top=z["top"], ff=z["ff"], shared_ff=z["shared_ff"])
+    cfg = S.stack_config(W, V, [layer] * z["layers"])
+    m = engine.StackModel(cfg, max_pos)
+
+    def mat(nm, r, c, std=None):
+        m.set_tensor(nm, _pool_bf16(S, r * c, std or 1.0 / np.sqrt(c), rng, pool).reshape(r, c))
+
+    def vec(nm, n, centre):
+        m.set_tensor(nm, S.to_bf16((centre + 0.05 * rng.standard_normal(n)).astype(np.float32)))
+
+    mat("embed", V, W, 1.0), mat("head", V, W), vec("embed.norm", W, 0.0), vec("final.norm", W, 0.0)
+    for i in range(z["layers"]):
+        p = f"l{i}."
+        qd, kd, vd, od = z["heads"] * z["dim"], z["kv_heads"] * z["dim"], z["kv_heads"] * z["vdim"], z["heads"] * z["vdim"]
+        mat(p + "mix.q", qd, W), mat(p + "mix.k", kd, W), mat(p + "mix.v", vd, W), mat(p + "mix.o", W, od)
+        vec(p + "mix.q.norm", qd, 1.0), vec(p + "mix.k.norm", kd, 1.0), vec(p + "norm1", W, 0.0), vec(p + "norm2", W, 0.0)
+        m.set_tensor(p + "mix.vmix", S.to_bf16(np.array(0.5, np.float32)))
+        mat(p + "mlp.router", z["experts"], W), vec(p + "mlp.router.b", z["experts"], 0.0)
+        for e in range(z["experts"]):
+            mat(p + f"mlp.e{e}.gate", z["ff"], W), mat(p + f"mlp.e{e}.up", z["ff"], W), mat(p + f"mlp.e{e}.down", W, z["ff"])
+        mat(p + "mlp.shared.gate", z["shared_ff"], W), mat(p + "mlp.shared.up", z["shared_ff"], W)
+        mat(p + "mlp.shared.down", W, z["shared_ff"])
+    m.finalize()
+    per_tok = (z["heads"] * z["dim"] + z["kv_heads"] * (z["dim"] + z["vdim"]) + z["heads"] * z["vdim"]) * W \
+        + 3 * W * (z["top"] * z["ff"] + z["shared_ff"]) + W * z["experts"]
+    return m, per_tok
+
+
+def _build_madalorn(S, engine, z, max_pos, rng, pool):
+    """Attention and delta-rule layers in turn (attention first), every layer with the routed feed-forward of the size."""
+    W, V, H, G, d = z["width"], z["vocab"], z["heads"], z["kv_heads"], z["dim"]
+    rank = d
+    att = S.madalorn_attention(H, G, d, window=z["window"], keep_first=64, base=250000.0,
+                               scaling={"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+    dl = S.madalorn_delta(H, G, d, d, conv=4)
+    moe = S.madalorn_moe(z["experts"], z["top"], z["ff"], shared_ff=z["shared_ff"], groups=4, keep=2)
+    layers = [S.madalorn_layer("attention" if i % 2 == 0 else "channel_delta", att if i % 2 == 0 else dl, moe)
+              for i in range(z["layers"])]
+    cfg = S.madalorn_config(W, V, layers)
+    shapes = {f"l{i}.mix.{n}": np.empty((rank, 0)) for i in range(z["layers"]) for n in ("a1", "g1")}
+    m = engine.StackModel(cfg, max_pos, shapes)
+
+    def mat(nm, r, c, std=None):
+        m.set_tensor(nm, _pool_bf16(S, r * c, std or 1.0 / np.sqrt(c), rng, pool).reshape(r, c))
+
+    def vec(nm, n, centre, spread=0.05):
+        m.set_tensor(nm, S.to_bf16((centre + spread * rng.standard_normal(n)).astype(np.float32)))
+
+    def norm(nm):
+        vec(nm, W, 1.0), vec(nm + ".b", W, 0.0)
+        m.set_tensor(nm + ".alpha", S.to_bf16(np.array(0.5, np.float32)))
+
+    mat("embed", V, W, 1.0), mat("head", V, W), norm("final.norm")
+    per_tok = 0
+    for i in range(z["layers"]):
+        p = f"l{i}."
+        norm(p + "norm1")
+        if i % 2 == 0:
+            mat(p + "mix.q", H * d, W), mat(p + "mix.k", G * d, W), mat(p + "mix.o", W, H * d), vec(p + "mix.pb", H, -2.0, 0.5)
+            per_tok += (H * d + G * d + H * d) * W
+        else:
+            mat(p + "mix.q", G * d, W), mat(p + "mix.k", G * d, W), mat(p + "mix.v", H * d, W), mat(p + "mix.o", W, H * d)
+            for n, c in (("q", G * d), ("k", G * d), ("v", H * d)):
+                mat(p + f"mix.{n}.conv", c, 4, 0.5)
+            mat(p + "mix.b", H, W), mat(p + "mix.a1", rank, W), mat(p + "mix.g1", rank, W)
+            mat(p + "mix.a2", H * d, rank), mat(p + "mix.g2", H * d, rank)
+            vec(p + "mix.A_log", H, -1.0, 0.3), vec(p + "mix.dt_bias", H * d, -1.0, 0.3), vec(p + "mix.norm", d, 1.0)
+            per_tok += (2 * G * d + 2 * H * d + H + 2 * rank) * W + 2 * H * d * rank
+        mat(p + "mlp.router", z["experts"], W)
+        for e in range(z["experts"]):
+            mat(p + f"mlp.e{e}.gate", z["ff"], W), mat(p + f"mlp.e{e}.up", z["ff"], W), mat(p + f"mlp.e{e}.down", W, z["ff"])
+        mat(p + "mlp.shared.gate", z["shared_ff"], W), mat(p + "mlp.shared.up", z["shared_ff"], W)
+        mat(p + "mlp.shared.down", W, z["shared_ff"]), mat(p + "mlp.shared.sg", 1, W)
+        per_tok += 3 * W * (z["top"] * z["ff"] + z["shared_ff"]) + W * (z["experts"] + 1)
+    m.finalize()
+    return m, per_tok / z["layers"]
+
+
 def stack_bench(args):
     from _pkg import load_package
     pkg = load_package()
@@ -127,61 +242,28 @@ def stack_bench(args):
     for name in [x for x in args.sizes.split(",") if x]:
         z = STACK_SIZES[name]
         W, V = z["width"], z["vocab"]
-        layer = S.stack_layer(z["heads"], z["kv_heads"], z["dim"], z["vdim"], z["window"], v_mix=True, experts=z["experts"],
-                              top=z["top"], ff=z["ff"], shared_ff=z["shared_ff"])
-        cfg = S.stack_config(W, V, [layer] * z["layers"])
         max_pos = T + args.steps + args.warmup + 64
-        m = engine.StackModel(cfg, max_pos)
-
-        def mat(nm, r, c, std=None):
-            m.set_tensor(nm, _pool_bf16(S, r * c, std or 1.0 / np.sqrt(c), rng, pool).reshape(r, c))
-
-        def vec(nm, n, centre):
-            m.set_tensor(nm, S.to_bf16((centre + 0.05 * rng.standard_normal(n)).astype(np.float32)))
-
+        if args.family == "madalorn":
+            # the delta rule's value size equals its key size here, and the attention's values are its keys
+            z = dict(z, vdim=z["dim"])
+            t0 = time.time()
+            m, per_tok = _build_madalorn(S, engine, z, max_pos, rng, pool)
+            r = {"size": name, "shape": z, "layers": "attention / channel_delta in turn", "load_s": round(time.time() - t0, 1)}
+            got, toks, first = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+            r.update(got)
+            m.free()
+            m, per_tok = _build_ralasun(S, engine, z, max_pos, rng, pool)
+            tw, _, _ = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+            m.free()
+            r["ralasun_twin"] = tw
+            results.append(r)
+            print(json.dumps(r), file=sys.stderr, flush=True)
+            continue
         t0 = time.time()
-        mat("embed", V, W, 1.0), mat("head", V, W), vec("embed.norm", W, 0.0), vec("final.norm", W, 0.0)
-        for i in range(z["layers"]):
-            p = f"l{i}."
-            qd, kd, vd, od = z["heads"] * z["dim"], z["kv_heads"] * z["dim"], z["kv_heads"] * z["vdim"], z["heads"] * z["vdim"]
-            mat(p + "mix.q", qd, W), mat(p + "mix.k", kd, W), mat(p + "mix.v", vd, W), mat(p + "mix.o", W, od)
-            vec(p + "mix.q.norm", qd, 1.0), vec(p + "mix.k.norm", kd, 1.0), vec(p + "norm1", W, 0.0), vec(p + "norm2", W, 0.0)
-            m.set_tensor(p + "mix.vmix", S.to_bf16(np.array(0.5, np.float32)))
-            mat(p + "mlp.router", z["experts"], W), vec(p + "mlp.router.b", z["experts"], 0.0)
-            for e in range(z["experts"]):
-                mat(p + f"mlp.e{e}.gate", z["ff"], W), mat(p + f"mlp.e{e}.up", z["ff"], W), mat(p + f"mlp.e{e}.down", W, z["ff"])
-            mat(p + "mlp.shared.gate", z["shared_ff"], W), mat(p + "mlp.shared.up", z["shared_ff"], W)
-            mat(p + "mlp.shared.down", W, z["shared_ff"])
-        m.finalize()
-        load_s = time.time() - t0
-        toks = rng.integers(0, V, T).astype(np.int32)
-        last_row = np.array([T - 1], np.int32)
-        r = {"size": name, "shape": z, "load_s": round(load_s, 1)}
-        per_tok = (z["heads"] * z["dim"] + z["kv_heads"] * (z["dim"] + z["vdim"]) + z["heads"] * z["vdim"]) * W \
-            + 3 * W * (z["top"] * z["ff"] + z["shared_ff"]) + W * z["experts"]
-        for terms, label in ((1, "bf16"), (3, "fp32_grade")):
-            m.set_prefill(terms, 1)
-            m.reset_kv()
-            m.prefill_rows(toks, 0, last_row)
-            best = 1e9
-            for _ in range(3):
-                m.reset_kv()
-                t0 = time.perf_counter()
-                m.prefill_rows(toks, 0, last_row)
-                best = min(best, time.perf_counter() - t0)
-            r[f"prefill_{label}_tokens_per_s"] = round(T / best, 1)
-            r[f"prefill_{label}_gemm_tflops"] = round(2.0 * T * per_tok * z["layers"] / best / 1e12, 2)
-        m.set_prefill(1, 1)
-        first = int(np.argmax(m.prefill_rows(toks, 0, last_row)[0]))  # the cache now holds T positions
-        m.generate_greedy(first, T, args.warmup)
-        t0 = time.perf_counter()
-        m.generate_greedy(first, T + args.warmup, args.steps)
-        dt = time.perf_counter() - t0
-        wb, kb = m.bytes_per_token(T + args.warmup)
-        r.update(decode_tokens_per_s=round(args.steps / dt, 1), decode_us_per_token=round(dt / args.steps * 1e6, 1),
-                 decode_bytes_per_token=int(wb + kb), decode_hbm_gbps=round((wb + kb) * args.steps / dt / 1e9, 1),
-                 decode_frac_of_hbm_peak=round((wb + kb) * args.steps / dt / 1e9 / HBM_PEAK_GBPS, 4),
-                 graph_nodes=m.graph_nodes())
+        m, per_tok = _build_ralasun(S, engine, z, max_pos, rng, pool)
+        r = {"size": name, "shape": z, "load_s": round(time.time() - t0, 1)}
+        got, toks, first = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+        r.update(got)
         m.free()
         # ---- the Llama twin ------------------------------------------------------------------------------------------
         lc = dict(hidden=W, inter=z["top"] * z["ff"] + z["shared_ff"], n_heads=z["heads"], n_kv_heads=z["kv_heads"],
@@ -218,9 +300,11 @@ def stack_bench(args):
             r["llama_twin"] = tw
         results.append(r)
         print(json.dumps(r), file=sys.stderr, flush=True)
-    print(json.dumps({"metric": "layer-list family (Ralasun): prefill / decode tokens/s beside a Llama model of equal size",
-                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "prefill_tokens": T, "dtype": "bf16 weights, "
-                      "fp32 activations", "data": "synthetic", "results": results}))
+    label = ("layer-list family (Madalorn): prefill / decode tokens/s beside a Ralasun model of equal size"
+             if args.family == "madalorn" else
+             "layer-list family (Ralasun): prefill / decode tokens/s beside a Llama model of equal size")
+    print(json.dumps({"metric": label, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "prefill_tokens": T,
+                      "dtype": "bf16 weights, fp32 activations", "data": "synthetic", "results": results}))
     return 0
 
 

@@ -88,10 +88,18 @@ __device__ __forceinline__ float row16_sum(float x) {
 }
 
 // E key channels per lane: dim <= 16 E. grid (vdim / 16 rounded up, heads), 256 threads.
+// The operands of 16 (8 for the largest key size) tokens at a time (k, q, g of the head; v of the workgroup's 16 columns; beta) are staged in LDS by
+// all threads together, the next stage's global loads in flight while the tokens of the stage in hand are walked: a token
+// then waits for an LDS read, not for a round trip to memory.
 template <int E>
 __global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) {
-  const int tid = threadIdx.x, sub = tid & 15;
-  const int col = blockIdx.x * 16 + (tid >> 4), h = blockIdx.y;
+  constexpr int DELTA_TB = E == 16 ? 8 : 16;  // tokens per stage (48 KB of LDS at most)
+  constexpr int DP = 16 * E;                 // padded key size
+  constexpr int NL = (DELTA_TB * DP) / 256;  // k / q / g elements a thread stages = E
+  __shared__ __attribute__((aligned(16))) float sk_[2][DELTA_TB][DP], sq_[2][DELTA_TB][DP], sg_[2][DELTA_TB][DP];
+  __shared__ float sv_[2][DELTA_TB][16], sb_[2][DELTA_TB];
+  const int tid = threadIdx.x, sub = tid & 15, cl = tid >> 4;
+  const int col = blockIdx.x * 16 + cl, h = blockIdx.y;
   const int kvh = h / (a.heads / a.kv_heads);
   const bool live = col < a.vdim;           // lanes of a column beyond vdim compute on zeros and store nothing
   const int d0 = sub * E;
@@ -103,44 +111,67 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const DeltaScanArgs a) 
   const float* kp = a.k + (size_t)kvh * a.dim;
   const float* gp = a.g + (size_t)h * a.dim;
   const int gd = a.heads * a.dim;
-  float kn[E], qn[E], gn[E], vn, bn;
-  auto load = [&](int t) __attribute__((always_inline)) {
+  // staging registers: element i of this thread is (token i * 256 + tid) / DP, channel (i * 256 + tid) % DP of the stage
+  float rk[NL], rq[NL], rg[NL], rv, rb;
+  auto fetch = [&](int t0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const bool in = d0 + e < a.dim;
-      kn[e] = in ? kp[(size_t)t * a.ldq + d0 + e] : 0.0f;
-      qn[e] = in ? qp[(size_t)t * a.ldq + d0 + e] : 0.0f;
-      gn[e] = in ? gp[(size_t)t * gd + d0 + e] : 0.0f;
+    for (int i = 0; i < NL; ++i) {
+      const int idx = i * 256 + tid, tt = idx / DP, d = idx % DP;
+      const bool in = t0 + tt < a.T && d < a.dim;
+      rk[i] = in ? kp[(size_t)(t0 + tt) * a.ldq + d] : 0.0f;
+      rq[i] = in ? qp[(size_t)(t0 + tt) * a.ldq + d] : 0.0f;
+      rg[i] = in ? gp[(size_t)(t0 + tt) * gd + d] : 0.0f;
     }
-    vn = live ? a.v[(size_t)t * a.ldv + (size_t)h * a.vdim + col] : 0.0f;
-    bn = a.beta[(size_t)t * a.heads + h];
+    const int tt = tid >> 4, c = blockIdx.x * 16 + (tid & 15);
+    rv = (tt < DELTA_TB && t0 + tt < a.T && c < a.vdim) ? a.v[(size_t)(t0 + tt) * a.ldv + (size_t)h * a.vdim + c] : 0.0f;
+    rb = (tid < DELTA_TB && t0 + tid < a.T) ? a.beta[(size_t)(t0 + tid) * a.heads + h] : 0.0f;
   };
-  load(0);
-  for (int t = 0; t < a.T; ++t) {
-    float kc[E], qc[E], gc[E];
+  auto stash = [&](int b) __attribute__((always_inline)) {
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      kc[e] = kn[e];
-      qc[e] = qn[e];
-      gc[e] = gn[e];
+    for (int i = 0; i < NL; ++i) {
+      const int idx = i * 256 + tid, tt = idx / DP, d = idx % DP;
+      sk_[b][tt][d] = rk[i];
+      sq_[b][tt][d] = rq[i];
+      sg_[b][tt][d] = rg[i];
     }
-    const float vc = vn, bc = bn;
-    if (t + 1 < a.T) load(t + 1);
-    float sk = 0.0f, sq = 0.0f, kq = 0.0f;
+    if ((tid >> 4) < DELTA_TB) sv_[b][tid >> 4][tid & 15] = rv;
+    if (tid < DELTA_TB) sb_[b][tid] = rb;
+  };
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  int b = 0;
+  for (int t0 = 0; t0 < a.T; t0 += DELTA_TB, b ^= 1) {
+    const bool more = t0 + DELTA_TB < a.T;
+    if (more) fetch(t0 + DELTA_TB);  // in flight under this stage's tokens
+    const int nt = a.T - t0 < DELTA_TB ? a.T - t0 : DELTA_TB;
+    for (int tt = 0; tt < nt; ++tt) {
+      float kc[E], qc[E], gc[E];
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      s[e] *= gc[e];
-      sk += s[e] * kc[e];
-      sq += s[e] * qc[e];
-      kq += kc[e] * qc[e];
+      for (int e = 0; e < E; ++e) {
+        kc[e] = sk_[b][tt][d0 + e];
+        qc[e] = sq_[b][tt][d0 + e];
+        gc[e] = sg_[b][tt][d0 + e];
+      }
+      const float vc = sv_[b][tt][cl], bc = sb_[b][tt];
+      float sk = 0.0f, sq = 0.0f, kq = 0.0f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        s[e] *= gc[e];
+        sk += s[e] * kc[e];
+        sq += s[e] * qc[e];
+        kq += kc[e] * qc[e];
+      }
+      sk = row16_sum(sk);
+      sq = row16_sum(sq);
+      kq = row16_sum(kq);
+      const float u = bc * (vc - sk);
+#pragma unroll
+      for (int e = 0; e < E; ++e) s[e] += kc[e] * u;
+      if (live && sub == 0) a.o[(size_t)(t0 + tt) * a.heads * a.vdim + (size_t)h * a.vdim + col] = sq + u * kq;
     }
-    sk = row16_sum(sk);
-    sq = row16_sum(sq);
-    kq = row16_sum(kq);
-    const float u = bc * (vc - sk);
-#pragma unroll
-    for (int e = 0; e < E; ++e) s[e] += kc[e] * u;
-    if (live && sub == 0) a.o[(size_t)t * a.heads * a.vdim + (size_t)h * a.vdim + col] = sq + u * kq;
+    if (more) stash(b ^ 1);  // the other buffer: its last readers passed the barrier at the end of the stage before
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
