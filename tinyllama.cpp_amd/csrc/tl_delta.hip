@@ -7,8 +7,8 @@
 // beta = sigmoid(.), g = exp(-exp(A_log[head]) * softplus(a + dt_bias)) per head and key channel. Everything that enters the
 // recurrence is FP32, and so is the state.
 //
-//   delta_pre    one workgroup per token: convolution (its last taps - 1 inputs of earlier calls come from a history that is
-//                part of the sequence's state), silu, the unit norms, beta and the decay.
+//   delta_pre    one workgroup per token and head: convolution (its last taps - 1 inputs of earlier calls come from a history
+//                that is part of the sequence's state), silu, the unit norms, beta and the decay.
 //   delta_scan   the recurrence. The columns of S (one per value channel) never mix: o_c = s_c . q, u_c = beta (v_c - s_c . k),
 //                s_c <- g * s_c + k u_c. Sixteen lanes share a column (each holds dim / 16 of its key channels in registers),
 //                four columns a wave, sixteen a workgroup, heads * vdim / 16 workgroups; the tokens are walked in order with
@@ -26,11 +26,25 @@ namespace {
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
 
-__global__ __launch_bounds__(256) void delta_pre_kernel(const DeltaPreArgs a) {
-  extern __shared__ float row[];  // [channels] silu(conv)
-  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+// grid (T, 2 * kv_heads + heads): a workgroup of 128 threads owns one head of one token -- a q head, a k head (convolution,
+// silu, unit norm), or a v head (convolution, silu) together with that head's decay channels and beta. One token (the decode
+// step) is thereby spread over as many workgroups as the layer has heads.
+__global__ __launch_bounds__(128) void delta_pre_kernel(const DeltaPreArgs a) {
+  __shared__ float red[2];
+  const int t = blockIdx.x, unit = blockIdx.y, tid = threadIdx.x;
   const int qd = a.kv_heads * a.dim, vd = a.heads * a.vdim, C = 2 * qd + vd, H = a.taps - 1;
-  for (int c = tid; c < C; c += 256) {
+  const bool is_v = unit >= 2 * a.kv_heads;
+  const int n = is_v ? a.vdim : a.dim;                                            // channels of this head
+  const int c0 = is_v ? 2 * qd + (unit - 2 * a.kv_heads) * a.vdim : unit * a.dim;  // its first channel
+  float* out = a.qkv + (size_t)t * C + c0;
+  float ss = 0.0f;
+  float y[4];  // n <= 512: four channels a thread
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int d = tid + 128 * r;
+    y[r] = 0.0f;
+    if (d >= n) continue;
+    const int c = c0 + d;
     const unsigned short* w = a.conv + (size_t)c * a.taps;
     float acc = 0.0f;
     for (int j = 0; j < a.taps; ++j) {
@@ -38,29 +52,32 @@ __global__ __launch_bounds__(256) void delta_pre_kernel(const DeltaPreArgs a) {
       const float in = tt >= 0 ? a.p[(size_t)tt * a.ld + c] : a.hist[(size_t)(H + tt) * C + c];
       acc += tl_bf2f(w[j]) * in;
     }
-    row[c] = acc * sigmoidf_(acc);
+    y[r] = acc * sigmoidf_(acc);
+    ss += y[r] * y[r];
     if (a.T == 1 && H > 0) {  // one token: this thread is the only reader of its channel's history, so it may shift it now
       for (int j = 0; j + 1 < H; ++j) a.hist[(size_t)j * C + c] = a.hist[(size_t)(j + 1) * C + c];
       a.hist[(size_t)(H - 1) * C + c] = a.p[c];
     }
   }
-  __syncthreads();
-  float* out = a.qkv + (size_t)t * C;
-  // q heads, then k heads: a wave per head
-  for (int hh = wave; hh < 2 * a.kv_heads; hh += 4) {
-    const float* x = row + (size_t)hh * a.dim;
-    float ss = 0.0f;
-    for (int d = lane; d < a.dim; d += 64) ss += x[d] * x[d];
+  float inv = 1.0f;
+  if (!is_v) {
     ss = tl_wave_sum(ss);
-    float inv = 1.0f / sqrtf(ss + 1e-6f);
-    if (hh < a.kv_heads) inv *= 1.0f / sqrtf((float)a.dim);
-    for (int d = lane; d < a.dim; d += 64) out[(size_t)hh * a.dim + d] = x[d] * inv;
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    inv = 1.0f / sqrtf(red[0] + red[1] + 1e-6f);
+    if (unit < a.kv_heads) inv *= 1.0f / sqrtf((float)a.dim);
   }
-  for (int c = 2 * qd + tid; c < C; c += 256) out[c] = row[c];
-  for (int h = tid; h < a.heads; h += 256) a.beta[(size_t)t * a.heads + h] = sigmoidf_(a.p[(size_t)t * a.ld + C + h]);
-  const int gd = a.heads * a.dim;
-  for (int c = tid; c < gd; c += 256) {
-    const float rate = expf(a.a_log[c / a.dim]);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int d = tid + 128 * r;
+    if (d < n) out[d] = y[r] * inv;
+  }
+  if (!is_v) return;
+  const int h = unit - 2 * a.kv_heads, gd = a.heads * a.dim;
+  if (tid == 0) a.beta[(size_t)t * a.heads + h] = sigmoidf_(a.p[(size_t)t * a.ld + C + h]);
+  const float rate = expf(a.a_log[h]);
+  for (int d = tid; d < a.dim; d += 128) {
+    const int c = h * a.dim + d;
     a.g[(size_t)t * gd + c] = expf(-rate * softplusf_(a.a[(size_t)t * gd + c] + a.dt_bias[c]));
   }
 }
@@ -204,8 +221,9 @@ int tl_launch_delta_pre(const DeltaPreArgs& a, hipStream_t s) {
   TL_REQUIRE(a.taps >= 1 && (a.taps == 1 || a.hist), "delta_pre: %d taps", a.taps);
   const int C = 2 * a.kv_heads * a.dim + a.heads * a.vdim;
   TL_REQUIRE(a.ld >= C + a.heads, "delta_pre: row stride %d below %d", a.ld, C + a.heads);
-  TL_REQUIRE(sizeof(float) * C <= 64 * 1024, "delta_pre: %d channels do not fit the staged row", C);
-  delta_pre_kernel<<<a.T, 256, sizeof(float) * C, s>>>(a);
+  TL_REQUIRE(a.dim <= 512 && a.vdim <= 512, "delta_pre: head sizes %d / %d above 512", a.dim, a.vdim);
+  TL_REQUIRE(2 * a.kv_heads + a.heads <= 65535, "delta_pre: too many heads");
+  delta_pre_kernel<<<dim3(a.T, 2 * a.kv_heads + a.heads), 128, 0, s>>>(a);
   if (a.T > 1 && a.taps > 1) conv_history_kernel<<<(C + 255) / 256, 256, 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;

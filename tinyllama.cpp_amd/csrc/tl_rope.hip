@@ -12,7 +12,7 @@
 //   unit norm  after the rotation each head is divided by its root mean square over dim (eps inside the root; no weights).
 //   caches     the finished keys go to row `pos` of the key cache; a design whose values are its keys as projected gets the
 //              untouched key row in the value cache in the same pass.
-// One workgroup per token, a wave per head in turn; a lane holds up to 4 pairs of a head (dim <= 512).
+// A wave per (token, head), four heads a workgroup; a lane holds up to 4 pairs of a head (dim <= 512).
 #include <math.h>
 
 #include <vector>
@@ -49,11 +49,12 @@ namespace {
 constexpr int kMaxPairs = 4;  // per lane: dim <= 512
 
 __global__ __launch_bounds__(256) void rotary_kernel(const RotaryArgs a) {
-  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
   const int pos = (a.pos_dev ? *a.pos_dev : a.start_pos) + t;
   const float fpos = (float)pos;
   const int kd = a.kv_heads * a.dim;
-  for (int hh = wave; hh < a.heads + a.kv_heads; hh += nwaves) {
+  // a wave per head: workgroup y of a token takes heads 4 y .. 4 y + 3 (one token of a decode step still fills several CUs)
+  for (int hh = blockIdx.y * 4 + (threadIdx.x >> 6); hh < a.heads + a.kv_heads; hh += 4 * gridDim.y) {
     float* x = a.qk + (size_t)t * a.ld + (size_t)hh * a.dim;
     const bool is_k = hh >= a.heads;
     const int kcol = (hh - a.heads) * a.dim;
@@ -102,7 +103,8 @@ __global__ __launch_bounds__(256) void rotary_kernel(const RotaryArgs a) {
     }
   }
   if (a.v_src)
-    for (int c = threadIdx.x; c < a.vd; c += blockDim.x) a.v_dst[(size_t)pos * a.vd + c] = a.v_src[(size_t)t * a.ld + c];
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < a.vd; c += blockDim.x * gridDim.y)
+      a.v_dst[(size_t)pos * a.vd + c] = a.v_src[(size_t)t * a.ld + c];
 }
 
 }  // namespace
@@ -116,7 +118,8 @@ int tl_launch_rotary(const RotaryArgs& a, hipStream_t s) {
   TL_REQUIRE(a.ld >= (a.heads + a.kv_heads) * a.dim, "rotary: row stride %d too short", a.ld);
   TL_REQUIRE(a.pos_dev || a.start_pos >= 0, "rotary: negative start position");
   TL_REQUIRE(!a.v_src || (a.v_dst && a.vd > 0), "rotary: a value row without its cache");
-  rotary_kernel<<<a.T, 256, 0, s>>>(a);
+  const int per_token = (a.heads + a.kv_heads + 3) / 4;
+  rotary_kernel<<<dim3(a.T, per_token < 65535 ? per_token : 65535), 256, 0, s>>>(a);
   TL_HIP(hipGetLastError());
   return 0;
 }

@@ -73,6 +73,12 @@ struct TlStack {
   int chunk = 2048;
   bool gemv_decode = true;
   bool fuse_router = true;  // TL_STACK_FUSE_ROUTER=0: the router as a launch of its own (A/B, tests)
+  // One token through a parallel block: mixer and feed-forward read the same h and meet only in the residual sum, so the
+  // feed-forward's launches go to a second stream (forked and joined by events; under capture they become a parallel branch
+  // of the graph) and the step's critical path per layer is the longer of the two chains, not their sum. TL_STACK_FORK=0: one stream.
+  bool fork = true;
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
   // workspaces for one chunk
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *proj = nullptr, *v_first = nullptr, *xn = nullptr;
   float* h = nullptr;       // norm-first blocks: the normalised input both sublayers read
@@ -242,7 +248,8 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
       CREATE_REQUIRE(sp.block == TL_BLOCK_PARALLEL, "tl_stack_create: layer %d: the delta rule runs in parallel blocks only", i);
       CREATE_REQUIRE(sp.conv_taps >= 1 && sp.conv_taps <= 64 && sp.decay_rank > 0 && sp.gate_rank > 0,
                      "tl_stack_create: layer %d: %d taps, inner sizes %d / %d", i, sp.conv_taps, sp.decay_rank, sp.gate_rank);
-      CREATE_REQUIRE(sp.dim <= 256, "tl_stack_create: layer %d: key size %d above 256", i, sp.dim);
+      CREATE_REQUIRE(sp.dim <= 256 && sp.vdim <= 512, "tl_stack_create: layer %d: key size %d above 256 or value size %d above 512", i,
+                     sp.dim, sp.vdim);
       L.qd = sp.kv_heads * sp.dim;  // queries share the keys' heads
       L.kd = sp.kv_heads * sp.dim;
       L.vd = sp.heads * sp.vdim;
@@ -336,6 +343,7 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
   if (const char* e = getenv("TL_STACK_CHUNK")) st->chunk = atoi(e) > 0 ? atoi(e) : st->chunk;
   if (const char* e = getenv("TL_STACK_GEMV")) st->gemv_decode = atoi(e) != 0;
   if (const char* e = getenv("TL_STACK_FUSE_ROUTER")) st->fuse_router = atoi(e) != 0;
+  if (const char* e = getenv("TL_STACK_FORK")) st->fork = atoi(e) != 0;
   *out = st;
   return 0;
 }
@@ -344,6 +352,9 @@ void tl_stack_free(TlStack* st) {
   if (!st) return;
   for (void* p : st->allocs) hipFree(p);
   hipFree(st->cache_base);
+  if (st->ev_fork) hipEventDestroy(st->ev_fork);
+  if (st->ev_join) hipEventDestroy(st->ev_join);
+  if (st->side) hipStreamDestroy(st->side);
   delete st;
 }
 
@@ -518,6 +529,15 @@ int tl_stack_finalize(TlStack* st, hipStream_t s) {
     TL_TRY(dev_alloc(st, &st->sgate, C));
     TL_TRY(dev_alloc(st, &st->sout, C * W));
     if (st->max_sff) TL_TRY(dev_alloc(st, &st->sact, C * st->max_sff));
+  }
+  bool any_parallel = false;
+  for (const Layer& L : st->layers) any_parallel |= L.sp.block == TL_BLOCK_PARALLEL && L.sp.mlp != TL_MLP_NONE;
+  if (st->fork && any_parallel) {
+    TL_HIP(hipStreamCreateWithFlags(&st->side, hipStreamNonBlocking));
+    TL_HIP(hipEventCreateWithFlags(&st->ev_fork, hipEventDisableTiming));
+    TL_HIP(hipEventCreateWithFlags(&st->ev_join, hipEventDisableTiming));
+  } else {
+    st->fork = false;
   }
   st->finalized = true;
   return tl_stack_reset(st, s);
@@ -863,17 +883,21 @@ int parallel_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
   const Layer& Wt = st->layers[L.wsrc];
   const tl_layer_spec& sp = L.sp;
   const int W = st->cfg.width;
-  if (sp.mixer == TL_MIXER_SWA) TL_TRY(swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s));
-  else TL_TRY(delta_mixer(st, L, Wt, st->h, T, s));
   ResidSumArgs r = {};
   r.x = st->x;
   r.T = T;
   r.width = W;
   r.a = st->proj;
   const bool one = T == 1 && st->gemv_decode;
+  const bool forked = st->fork && T == 1 && sp.mlp != TL_MLP_NONE;
+  hipStream_t fs = forked ? st->side : s;  // the feed-forward's stream
+  if (forked) {
+    TL_HIP(hipEventRecord(st->ev_fork, s));
+    TL_HIP(hipStreamWaitEvent(st->side, st->ev_fork, 0));
+  }
   if (sp.mlp == TL_MLP_MOE) {
-    TL_TRY(tl_launch_router(router_args(st, L, Wt, st->h, T), s));
-    TL_TRY(moe_experts(st, L, Wt, st->h, T, st->sout, s));
+    TL_TRY(tl_launch_router(router_args(st, L, Wt, st->h, T), fs));
+    TL_TRY(moe_experts(st, L, Wt, st->h, T, st->sout, fs));
     if (one) {
       r.b = st->sout;  // experts and shared expert already summed (the gate applied)
     } else {
@@ -899,7 +923,7 @@ int parallel_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
       d.up_add = sp.glu_up_add;
       d.act = st->act_buf;
       d.y = st->sout;
-      TL_TRY(tl_launch_moe_decode(d, s));
+      TL_TRY(tl_launch_moe_decode(d, fs));
     } else {
       DenseArgs u = {};
       u.w = Wt.sgu;
@@ -915,11 +939,15 @@ int parallel_layer(TlStack* st, size_t li, int T, int start_pos, const int* pos_
       u.glu_limit = sp.shared_limit;
       u.glu_alpha = sp.act_alpha;
       u.glu_up_add = sp.glu_up_add;
-      TL_TRY(tl_launch_dense_gemm(u, s));
-      TL_TRY(project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, s));
+      TL_TRY(tl_launch_dense_gemm(u, fs));
+      TL_TRY(project(st, Wt.sdown, W, ff, st->sact, ff, st->sout, W, T, fs));
     }
     r.b = st->sout;
   }
+  if (forked) TL_HIP(hipEventRecord(st->ev_join, st->side));
+  if (sp.mixer == TL_MIXER_SWA) TL_TRY(swa_mixer(st, L, Wt, st->h, T, start_pos, pos_dev, s));
+  else TL_TRY(delta_mixer(st, L, Wt, st->h, T, s));
+  if (forked) TL_HIP(hipStreamWaitEvent(s, st->ev_join, 0));
   if (li + 1 < st->layers.size() && st->layers[li + 1].sp.block == TL_BLOCK_PARALLEL) {
     r.next = dyt_of_layer(st->layers[st->layers[li + 1].wsrc]);
     r.h = st->h;
