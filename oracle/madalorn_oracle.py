@@ -153,7 +153,9 @@ class MadalornOracle:
         self.pos = 0
 
     def src(self, i):
-        return self.c["layers"][i].get("weights_of", i)
+        while "weights_of" in self.c["layers"][i]:
+            i = self.c["layers"][i]["weights_of"]
+        return i
 
     def norm(self, name, x):
         return dyt(x, self.w[name + ".alpha"].reshape(()), self.w[name], self.w[name + ".b"])

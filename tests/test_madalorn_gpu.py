@@ -39,7 +39,9 @@ def small_config(synth, variant="mixed"):
             L("channel_delta", D(4, 2, 16, 12, conv=3), M(6, 2, 24, shared_ff=40, groups=3, keep=2), weights_of=1),
             L("attention", A(2, 2, 36, window=None, rot_dims=36, base=500.0), None),
             L("channel_delta", D(2, 2, 20, 8, conv=2), {"kind": "dense", "ff": 24}),
-            L("attention", A(6, 3, 20, window=17, keep_first=0, rot_dims=8), M(5, 5, 8, shared_ff=0, groups=1, keep=1))], softcap=11.0)
+            L("attention", A(6, 3, 20, window=17, keep_first=0, rot_dims=8), M(5, 5, 8, shared_ff=0, groups=1, keep=1)),
+            L("attention", A(4, 2, 24, window=9, keep_first=3, rot_dims=16, scaling=ext), {"kind": "dense", "ff": 40}, weights_of=2)],
+            softcap=11.0)  # (the last layer borrows from a layer that borrows)
     if variant == "odd":  # nothing divisible by 4: every scalar fallback path; the recurrent layer first
         return synth.madalorn_config(37, 53, [
             L("channel_delta", D(3, 3, 5, 7, conv=5), M(4, 1, 5, shared_ff=7, groups=4, keep=1)),

@@ -188,9 +188,9 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
                    "runs in parallel blocks only", i);
     L.wsrc = i;
     if (sp.weights_of > 0) {
-      L.wsrc = sp.weights_of - 1;
-      CREATE_REQUIRE(L.wsrc < i && st->layers[L.wsrc].wsrc == L.wsrc, "tl_stack_create: layer %d takes its tensors from layer %d, "
-                     "which is not an earlier layer with tensors of its own", i, L.wsrc);
+      CREATE_REQUIRE(sp.weights_of - 1 < i, "tl_stack_create: layer %d takes its tensors from layer %d, which is not an earlier "
+                     "layer", i, sp.weights_of - 1);
+      L.wsrc = st->layers[sp.weights_of - 1].wsrc;  // (a layer that itself borrows hands on the owner)
       tl_layer_spec a = sp, b = st->layers[L.wsrc].sp;
       a.weights_of = b.weights_of = 0;
       CREATE_REQUIRE(memcmp(&a, &b, sizeof(a)) == 0, "tl_stack_create: layer %d differs from layer %d whose tensors it uses", i, L.wsrc);

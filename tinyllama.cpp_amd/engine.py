@@ -452,10 +452,12 @@ def _ralasun_spec(sp, i, L):
             sp.shared_ff, sp.shared_limit = sh["ff"], float(sh["limit"])
 
 
-def _madalorn_spec(sp, i, L, tensors):
+def _madalorn_spec(sp, i, L, tensors, layers):
     mx, ml = L["mixer"], L.get("mlp")
-    src = L.get("weights_of", i)
-    sp.weights_of = src + 1 if "weights_of" in L else 0
+    src = i
+    while "weights_of" in layers[src]:
+        src = layers[src]["weights_of"]
+    sp.weights_of = L["weights_of"] + 1 if "weights_of" in L else 0
     sp.block, sp.heads, sp.kv_heads, sp.dim, sp.vdim = 1, mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
     sp.act_alpha, sp.glu_up_add, sp.expert_limit, sp.shared_limit = 1.0, 0.0, float("inf"), float("inf")
     if L["type"] == "attention":
@@ -497,7 +499,7 @@ def stack_config_struct(config, max_pos, tensors=None):
     madalorn = config.get("architecture") == "Madalorn"
     for i, L in enumerate(layers):
         if madalorn:
-            _madalorn_spec(arr[i], i, L, tensors or {})
+            _madalorn_spec(arr[i], i, L, tensors or {}, layers)
         else:
             _ralasun_spec(arr[i], i, L)
     c = capi.StackConfig(config["width"], config["vocab"], len(layers), int(max_pos), float(config["norm"]["eps"]), arr,

@@ -90,7 +90,8 @@ int tensor_rows(const SafeTensorsFile& file, const std::string& name) {
   return (int)t->shape[0];
 }
 
-tl_layer_spec madalorn_layer(const Json& L, int index, const SafeTensorsFile& file) {
+tl_layer_spec madalorn_layer(const Json& layers, int index, const SafeTensorsFile& file) {
+  const Json& L = layers.arr[index];
   const std::string where = "layers[" + std::to_string(index) + "]";
   tl_layer_spec sp = {};
   const std::string& type = L.at("type").as_string("type");
@@ -100,6 +101,11 @@ tl_layer_spec madalorn_layer(const Json& L, int index, const SafeTensorsFile& fi
     src = (int)wo->as_int("weights_of");
     if (src < 0 || src >= index) throw std::runtime_error(where + ": weights_of must name an earlier layer");
     sp.weights_of = src + 1;
+    while (const Json* more = present(layers.arr[src], "weights_of")) {  // the owner of the tensors, for the sizes shapes give
+      const int next = (int)more->as_int("weights_of");
+      if (next < 0 || next >= src) throw std::runtime_error(where + ": weights_of must name an earlier layer");
+      src = next;
+    }
   }
   sp.block = TL_BLOCK_PARALLEL;
   sp.heads = geti(mx, "heads");
@@ -183,7 +189,7 @@ void load_stack_folder(const std::string& dir, int device, int max_context, Load
   file.open(dir + "/model.safetensors");
   std::vector<tl_layer_spec> specs;
   for (size_t i = 0; i < layers.arr.size(); ++i)
-    specs.push_back(madalorn ? madalorn_layer(layers.arr[i], (int)i, file) : ralasun_layer(layers.arr[i], (int)i, file));
+    specs.push_back(madalorn ? madalorn_layer(layers, (int)i, file) : ralasun_layer(layers.arr[i], (int)i, file));
   tl_stack_config sc = {};
   sc.width = geti(cfg, "width");
   sc.vocab = geti(cfg, "vocab");

@@ -385,7 +385,7 @@ def build_madalorn(config, seed=0, gain=1.0, ranks=(8, 8)):
     def norm(name):
         vec(name, W, 1.0, 0.1)
         vec(name + ".b", W, 0.0, 0.05)
-        t[name + ".alpha"] = to_bf16(np.array(rng.uniform(0.4, 0.9), np.float32))
+        t[name + ".alpha"] = to_bf16(np.array(rng.uniform(0.4, 0.9), np.float32)).reshape(())  # a scalar tensor: shape []
 
     def glu(p, ff):
         mat(p + "gate", ff, W, 2.0 / np.sqrt(W))
@@ -446,10 +446,11 @@ def write_stack_dir(path, config, tensors):
         json.dump(config, f, indent=1)
     header, off, blobs = {}, 0, []
     for name, a in tensors.items():
+        shape = list(np.shape(a))  # (a scalar tensor keeps its empty shape)
         a = np.ascontiguousarray(a)
         dt = {np.dtype(np.uint16): "BF16", np.dtype(np.float32): "F32", np.dtype(np.int32): "I32"}[a.dtype]
         b = a.tobytes()
-        header[name] = {"dtype": dt, "shape": list(a.shape), "data_offsets": [off, off + len(b)]}
+        header[name] = {"dtype": dt, "shape": shape, "data_offsets": [off, off + len(b)]}
         off += len(b)
         blobs.append(b)
     h = json.dumps(header, separators=(",", ":")).encode()
