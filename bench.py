@@ -59,6 +59,7 @@ def parse():
                          "equal size (one GPU; prints its own JSON line; the default workload and line are untouched)")
     ap.add_argument("--sizes", default="s,m,l", help="with --family: comma-separated names out of s, m, l")
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="with --family: prompt length of the prefill leg")
+    ap.add_argument("--no-twin", action="store_true", help="with --family: only the family's own model (for kernel profiles)")
     return ap.parse_args()
 
 
@@ -252,10 +253,11 @@ def stack_bench(args):
             got, toks, first = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
             r.update(got)
             m.free()
-            m, per_tok = _build_ralasun(S, engine, z, max_pos, rng, pool)
-            tw, _, _ = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
-            m.free()
-            r["ralasun_twin"] = tw
+            if not args.no_twin:
+                m, per_tok = _build_ralasun(S, engine, z, max_pos, rng, pool)
+                tw, _, _ = _time_stack_model(m, args, T, V, z["layers"], per_tok, rng)
+                m.free()
+                r["ralasun_twin"] = tw
             results.append(r)
             print(json.dumps(r), file=sys.stderr, flush=True)
             continue
@@ -268,7 +270,7 @@ def stack_bench(args):
         # ---- the Llama twin ------------------------------------------------------------------------------------------
         lc = dict(hidden=W, inter=z["top"] * z["ff"] + z["shared_ff"], n_heads=z["heads"], n_kv_heads=z["kv_heads"],
                   n_layers=z["layers"], vocab=V, max_pos=max_pos, eps=1e-5, rope_theta=10000.0)
-        if W // z["heads"] == z["dim"] and z["dim"] == z["vdim"]:
+        if W // z["heads"] == z["dim"] and z["dim"] == z["vdim"] and not args.no_twin:
             lm = engine.Model(lc)
             for nm, typ, rows, cols in S.tensor_plan(lc, "q8_0"):
                 lm.set_tensor(nm, typ, S.make_tensor(nm, typ, rows, cols, 42), rows, cols)
