@@ -525,3 +525,90 @@ def test_generation_through_the_host_session(env, tmp_path):
     synth.write_stack_dir(str(tmp_path / "bad"), bad, tensors)
     with pytest.raises(hostapi.TlHostError, match="weights_of"):
         hostapi.Session(str(tmp_path / "bad"), 0, 64)
+
+
+def random_config(synth, seed):
+    """A configuration drawn at random: layer order, head counts and ratios, head sizes (also indivisible by 4 and above
+    128), windows shorter and longer than the prompt, kept keys beyond the window, rotation on part of a head or none,
+    extension or none, taps, expert / group / top combinations, borrowed tensors, with and without a cap."""
+    rng = np.random.default_rng(1000 + seed)
+    A, D, M, L = synth.madalorn_attention, synth.madalorn_delta, synth.madalorn_moe, synth.madalorn_layer
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+
+    def mlp():
+        kind = pick(["dense", "moe", "moe", None])
+        if kind is None:
+            return None
+        if kind == "dense":
+            return {"kind": "dense", "ff": int(pick([7, 16, 40, 100]))}
+        groups = int(pick([1, 2, 3, 4]))
+        per = int(pick([1, 2, 3, 5]))
+        keep = int(rng.integers(1, groups + 1))
+        top = int(rng.integers(1, keep * per + 1))
+        return M(groups * per, top, int(pick([6, 16, 33])), shared_ff=int(pick([0, 12, 48])), groups=groups, keep=keep)
+
+    def mixer(kind):
+        if kind == "attention":
+            G = int(pick([1, 2, 3]))
+            H = G * int(pick([1, 2, 4]))
+            d = int(pick([6, 10, 16, 32, 48, 64, 136]))
+            window = pick([None, 1, 2, 7, 33, 64, 100, 1000])
+            keep = int(pick([0, 1, 5, 40, 90]))
+            rot = int(pick([0, 2, d // 2 * 2, max(2, d // 4 * 2)]))
+            sc = pick([None, {"factor": float(pick([2.0, 8.0, 1.0])), "original": int(pick([16, 64, 4096])),
+                              "fast": float(pick([1.0, 4.0, 32.0])), "slow": float(pick([0.25, 1.0]))}])
+            m = A(H, G, d, window=window, keep_first=keep, rot_dims=rot, base=float(pick([100.0, 10000.0, 5e5])), scaling=sc,
+                  scale=float(pick([0.1, d ** -0.5, 0.5])))
+            if rot == 0:
+                del m["rot"]
+            return m
+        G = int(pick([1, 2, 3]))
+        H = G * int(pick([1, 2, 3]))
+        return D(H, G, int(pick([3, 8, 16, 24, 64, 130])), int(pick([1, 5, 16, 40, 72])), conv=int(pick([1, 2, 3, 4, 6])))
+
+    layers = []
+    for i in range(int(rng.integers(2, 7))):
+        if layers and rng.random() < 0.3:
+            j = int(rng.integers(0, len(layers)))
+            layers.append(dict(layers[j], weights_of=j))
+            continue
+        kind = pick(["attention", "channel_delta"])
+        layers.append(L(kind, mixer(kind), mlp()))
+    cfg = synth.madalorn_config(int(pick([24, 50, 64, 100])), int(pick([40, 97, 130])), layers, eps=float(pick([1e-6, 1e-5, 1e-2])),
+                                softcap=float(pick([8.0, 30.0, 50.0])))
+    if rng.random() < 0.25:
+        del cfg["logit_softcap"]
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random(env, seed, tmp_path):
+    """Through the host session over a checkpoint folder (so the configuration reader is part of what is tested): a prompt in
+    portions and decoded tokens against the oracle, twice over so that state and cache are given back in between."""
+    from tinyllama_cpp_amd import hostapi
+    synth = env["synth"]
+    cfg = random_config(synth, seed)
+    tensors = synth.build_madalorn(cfg, seed, ranks=(3 + seed % 5, 2 + seed % 7))
+    synth.write_stack_dir(str(tmp_path / "ckpt"), cfg, tensors)
+    orc = env["oracle"].MadalornOracle(cfg, tensors)
+    rng = np.random.default_rng(seed)
+    n = 150
+    s = hostapi.Session(str(tmp_path / "ckpt"), 0, n)
+    s.set_exact(True)
+    for _ in range(2):
+        toks = rng.integers(0, cfg["vocab"], n).astype(np.int32)
+        orc.reset()
+        want = orc.forward(list(toks))
+        s.reset()
+        got, p = [], 0
+        for size in [int(x) for x in rng.integers(1, 24, 6)] + [2]:
+            got.append(s.forward(toks[p:p + size], p, list(range(size))))
+            p += size
+        got += [s.forward(toks[i:i + 1], i, [0]) for i in range(p, n)]
+        assert rel_rms(np.concatenate(got), want) < FP32_TOL, json_of(cfg)
+    s.close()
+
+
+def json_of(cfg):
+    import json
+    return json.dumps(cfg)
