@@ -344,7 +344,8 @@ int tl_moe_route_groups(const float* x_dev, int num_tokens, int width, const voi
 int tl_dyt_norm(const float* x_dev, const float* alpha_dev, const float* weight_dev, const float* bias_dev, float* out_dev,
                 int num_tokens, int width, void* stream);
 /* rotary positions as tl_layer_spec describes them (rot_factor <= 0: plain frequencies), in place on x [T][heads * dim] at
- * positions start_pos.., then (unit_norm != 0) every head divided by its root mean square (eps inside the root) */
+ * positions start_pos.., then (unit_norm != 0) every head divided by its root mean square (eps inside the root). The
+ * frequencies and the product position * frequency are double; cos and sin of its remainder in [-pi, pi] are FP32. */
 int tl_rotary_heads(float* x_dev, int num_tokens, int start_pos, int heads, int dim, int rot_dims, float rot_base,
                     float rot_factor, float rot_original, float rot_fast, float rot_slow, int unit_norm, float eps, void* stream);
 /* what precedes the gated delta rule, per token: p [T][ld] holds the projections q (kv_heads * dim) | k (kv_heads * dim) |

@@ -2,7 +2,9 @@
 //
 //   rotation   on the first rot_dims dimensions of each head, dimension 2i paired with 2i + 1 (the interleaved layout):
 //              (u, v) at position p -> (u cos a - v sin a, v cos a + u sin a), a = p * f_i, f_i = base^(-2i / rot_dims).
-//              Position, angle, cos and sin are FP32 on the device.
+//              The angle is formed in double (an integer position times a double frequency) and brought into [-pi, pi]
+//              there; cos and sin of that remainder are FP32. An FP32 product p * f_i alone is off by up to p * 2^-24
+//              radians, which at a few thousand positions is what decides the error of the logits.
 //   extension  (factor > 0) the frequencies of slowly turning pairs are divided by `factor`, fast ones stay, with a linear
 //              ramp between the pair that makes `fast` turns and the one that makes `slow` turns over the original context:
 //              d(t) = rot_dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(d(fast)), 0),
@@ -19,7 +21,7 @@
 
 #include "tl_stack.h"
 
-void tl_rotary_frequencies(int rot_dims, double base, double factor, double original, double fast, double slow, float* f,
+void tl_rotary_frequencies(int rot_dims, double base, double factor, double original, double fast, double slow, double* f,
                            float* mscale) {
   const int half = rot_dims / 2;
   const double pi = 3.14159265358979323846;
@@ -39,7 +41,7 @@ void tl_rotary_frequencies(int rot_dims, double base, double factor, double orig
       r = r < 0.0 ? 0.0 : r > 1.0 ? 1.0 : r;
       fi = fi / factor * r + fi * (1.0 - r);
     }
-    f[i] = (float)fi;
+    f[i] = fi;
   }
   *mscale = factor > 0.0 ? (float)(0.1 * log(factor) + 1.0) : 1.0f;
 }
@@ -51,7 +53,7 @@ constexpr int kMaxPairs = 4;  // per lane: dim <= 512
 __global__ __launch_bounds__(256) void rotary_kernel(const RotaryArgs a) {
   const int t = blockIdx.x, lane = threadIdx.x & 63;
   const int pos = (a.pos_dev ? *a.pos_dev : a.start_pos) + t;
-  const float fpos = (float)pos;
+  const double dpos = (double)pos;
   const int kd = a.kv_heads * a.dim;
   // a wave per head: workgroup y of a token takes heads 4 y .. 4 y + 3 (one token of a decode step still fills several CUs)
   for (int hh = blockIdx.y * 4 + (threadIdx.x >> 6); hh < a.heads + a.kv_heads; hh += 4 * gridDim.y) {
@@ -71,7 +73,8 @@ __global__ __launch_bounds__(256) void rotary_kernel(const RotaryArgs a) {
         if (d1 < a.dim) vr[d1] = v[r];
       }
       if (d1 < a.rot_dims) {
-        const float ang = fpos * a.freq[i];
+        const double full = dpos * a.freq[i];
+        const float ang = (float)(full - 6.283185307179586476925 * rint(full * 0.159154943091895335769));
         float sn, cs;
         sincosf(ang, &sn, &cs);
         sn *= a.mscale;
@@ -129,15 +132,15 @@ extern "C" int tl_rotary_heads(float* x_dev, int num_tokens, int start_pos, int 
                                void* stream) {
   TL_REQUIRE(rot_dims >= 0 && rot_dims <= dim && (rot_dims & 1) == 0, "tl_rotary_heads: %d rotating dimensions of %d", rot_dims, dim);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  std::vector<float> f(rot_dims / 2 + 1);
+  std::vector<double> f(rot_dims / 2 + 1);
   float mscale = 1.0f;
-  float* fdev = nullptr;
+  double* fdev = nullptr;
   if (rot_dims > 0) {
     tl_rotary_frequencies(rot_dims, rot_base, rot_factor, rot_original, rot_fast, rot_slow, f.data(), &mscale);
     void* ws = nullptr;
-    TL_TRY(tl_scratch(TL_SCRATCH_ROTARY, sizeof(float) * (rot_dims / 2), &ws));
-    fdev = static_cast<float*>(ws);
-    TL_HIP(hipMemcpyAsync(fdev, f.data(), sizeof(float) * (rot_dims / 2), hipMemcpyHostToDevice, s));
+    TL_TRY(tl_scratch(TL_SCRATCH_ROTARY, sizeof(double) * (rot_dims / 2), &ws));
+    fdev = static_cast<double*>(ws);
+    TL_HIP(hipMemcpyAsync(fdev, f.data(), sizeof(double) * (rot_dims / 2), hipMemcpyHostToDevice, s));
     TL_HIP(hipStreamSynchronize(s));
   }
   RotaryArgs a = {};

@@ -176,13 +176,13 @@ int tl_launch_moe_decode(const MoeDecodeArgs& a, hipStream_t s);
 
 // ---- tl_rope.hip -------------------------------------------------------------------------------------------------------
 // f[i] (i < rot_dims / 2) and the factor on cos / sin of a layer's rotary positions (tl_layer_spec: rot_*), computed in double
-void tl_rotary_frequencies(int rot_dims, double base, double factor, double original, double fast, double slow, float* f,
+void tl_rotary_frequencies(int rot_dims, double base, double factor, double original, double fast, double slow, double* f,
                            float* mscale);
 struct RotaryArgs {
   float* qk;             // [T][ld]: q heads (heads * dim) | k heads (kv_heads * dim) of a token, updated in place
   int ld, heads, kv_heads, dim;
   int rot_dims;          // the first rot_dims dimensions of a head rotate: (2i, 2i + 1) by position * freq[i]
-  const float* freq;     // device [rot_dims / 2]
+  const double* freq;    // device [rot_dims / 2], double: position * frequency is formed and reduced to [-pi, pi] in double
   float mscale;          // on cos and sin
   int unit_norm;         // 1: after the rotation a head is divided by its root mean square (eps inside the root)
   float eps;

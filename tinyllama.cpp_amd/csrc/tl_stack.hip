@@ -45,7 +45,8 @@ struct Layer {
   uint16_t *wqkv = nullptr, *wo = nullptr;
   float *q_norm = nullptr, *k_norm = nullptr, *lambda = nullptr, *norm1 = nullptr, *norm2 = nullptr;
   float *norm1_b = nullptr, *norm1_alpha = nullptr;  // Dynamic Tanh
-  float *pb = nullptr, *freq = nullptr;              // sigmoid bias per head; rotary frequencies
+  float* pb = nullptr;                               // sigmoid bias per head
+  double* freq = nullptr;                            // rotary frequencies
   float mscale = 1.0f;
   uint16_t *wa2 = nullptr, *wg2 = nullptr, *conv = nullptr;  // delta rule
   float *a_log = nullptr, *dt_bias = nullptr, *onorm = nullptr;
@@ -235,10 +236,10 @@ int tl_stack_create(const tl_stack_config* cfg, TlStack** out) {
         if ((rc = dev_alloc(st, &L.lambda, 1))) break;
         if ((rc = dev_alloc(st, &L.pb, sp.heads))) break;
         if (sp.rot_dims > 0) {
-          std::vector<float> f(sp.rot_dims / 2);
+          std::vector<double> f(sp.rot_dims / 2);
           tl_rotary_frequencies(sp.rot_dims, sp.rot_base, sp.rot_factor, sp.rot_original, sp.rot_fast, sp.rot_slow, f.data(), &L.mscale);
           if ((rc = dev_alloc(st, &L.freq, f.size()))) break;
-          if (hipMemcpy(L.freq, f.data(), sizeof(float) * f.size(), hipMemcpyHostToDevice) != hipSuccess) {
+          if (hipMemcpy(L.freq, f.data(), sizeof(double) * f.size(), hipMemcpyHostToDevice) != hipSuccess) {
             tl_set_error("tl_stack_create: upload of the rotary frequencies failed");
             return fail(1);
           }
